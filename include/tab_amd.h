@@ -1,0 +1,106 @@
+/*
+ * tab_amd.h - C ABI of the MI355X (gfx950) TAB quantize + bitwise-convolution library.
+ *
+ * All pointers named dev_* are device (HBM) addresses on the current HIP device; the
+ * library never copies to or from the host.  `stream` is a hipStream_t passed as void*
+ * (NULL = the default stream).  Every call only enqueues work on `stream` and returns
+ * without synchronising.  Functions returning int give TAB_OK or a negative
+ * tab_status; tab_status_string() names it and tab_last_error() holds a longer message
+ * for the calling thread.
+ *
+ * Data layouts are the reference's (ntuliuteam/TAB):
+ *   X    fp32  [N][H][W][C]                                  TAB_GEMM.cu:163-208
+ *   QX   int64 [N][H][W][PC][bits], PC = ceil(C/64), channel c -> word c/64, bit c%64
+ *        (LSB first); bits = 2: plane 0 = sign marker, plane 1 = nonzero marker;
+ *        bits = 1: bit set <=> value -1                     TAB_GEMM.cu:196-197,238,321
+ *   QW   the same layout with (N,H,W,C) = (KN,KH,KW,C)
+ *   Y    fp32  [N*OH*OW][KN]  (labelled (N,KN,OH,OW) by the caller)   TAB_GEMM.cu:53,526
+ */
+#ifndef TAB_AMD_H
+#define TAB_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum tab_status {
+    TAB_OK = 0,
+    TAB_ERR_BAD_ARGUMENT = -1, /* NULL pointer, non-positive extent, bad type/bitwidth */
+    TAB_ERR_BAD_SHAPE = -2,    /* empty output, or a size that overflows the index range */
+    TAB_ERR_WORKSPACE = -3,    /* workspace missing or smaller than required */
+    TAB_ERR_DEVICE = -4        /* a HIP call failed; see tab_last_error() */
+} tab_status;
+
+/* Conv types, TAB_GPU.cpp:27 ("0: TNN, 1, TBN, 2: BTN, 3: BNN"): first letter =
+ * activation precision, second = weight precision. */
+enum { TAB_TNN = 0, TAB_TBN = 1, TAB_BTN = 2, TAB_BNN = 3 };
+
+const char *tab_status_string(int status);
+const char *tab_last_error(void);
+/* "tab_amd <version> gfx950"; lets a binding check what it loaded. */
+const char *tab_version(void);
+
+/* PC = ceil(C/64) (TAB_GEMM.cu:262-265). */
+int tab_packed_channels(int C);
+
+/* Output extent (in + 2*pad - k + 1) / stride, integer division (TAB_GEMM.cu:354-357). */
+int tab_out_extent(int in, int pad, int k, int stride);
+
+/*
+ * Replaces QuanWithCuda_TAB (TAB_GEMM.cu:250-322), the body of
+ * TAB_Quantize(X, thresholds, bitwidth, N, H, W, C) (TAB_GPU.cpp:53-58).
+ *   dev_X    fp32 [N*H*W*C]
+ *   dev_ths  fp32 [>=N], threshold of item n is ths[n] (TAB_CPU.cpp:67,72)
+ *   bitwidth 2: ternarize (v > t -> +1, else v < -t -> -1, else 0); 1: binarize (v < t -> -1)
+ *   dev_QX   int64 [N*H*W*PC*bitwidth], every element is written
+ *   dev_BTN  int32 [N]; bitwidth 2: popcount of item n's nonzero plane (TAB_GEMM.cu:150-160,
+ *            for every n); bitwidth 1: zeros (TAB_GEMM.cu:283)
+ */
+int tab_quantize(const float *dev_X, const float *dev_ths, int bitwidth, int N, int H, int W,
+                 int C, int64_t *dev_QX, int32_t *dev_BTN, void *stream);
+
+/*
+ * Bytes of device scratch tab_conv2d needs for the packed activation
+ * (the reference cudaMallocs pad_a/img_a per call, TAB_GEMM.cu:391-397).  0 on bad arguments.
+ */
+size_t tab_conv2d_workspace_bytes(int type, int N, int H, int W, int C);
+
+/*
+ * Replaces ConvWithCuda_TAB (TAB_GEMM.cu:325-527), the body of
+ * TAB_Conv2d(X, QW, thresholds, btn, type, padding1, padding2, stride1, stride2,
+ *            N, H, W, C, KN, KH, KW) (TAB_GPU.cpp:34-42).
+ *   dev_X   fp32 [N*H*W*C]; quantized on the fly: ternary for TNN/TBN, binary for BTN/BNN
+ *           (TAB_GEMM.cu:419-426)
+ *   dev_QW  int64 [KN*KH*KW*PC*wbits], wbits = 2 for TNN/BTN, 1 for TBN/BNN (374-379)
+ *   dev_ths fp32 [>=N]
+ *   dev_btn int32 [>=KN], read only for BTN (TAB_GEMM.cu:116); may be NULL otherwise
+ *   dev_Y   fp32 [N*OH*OW*KN], OH = tab_out_extent(H, padding1, KH, stride1), OW likewise;
+ *           every element is written
+ *   workspace / workspace_bytes: device scratch of at least tab_conv2d_workspace_bytes()
+ *           bytes, 16-byte aligned; owned by the caller, reusable once the stream has
+ *           passed this call
+ * Padded taps read all-zero words: value 0 for ternary, +1 for binary activations
+ * (TAB_CPU.cpp:39,155); BNN's constant is KH*KW*C (TAB_GEMM.cu:509).
+ */
+int tab_conv2d(const float *dev_X, const int64_t *dev_QW, const float *dev_ths,
+               const int32_t *dev_btn, int type, int padding1, int padding2, int stride1,
+               int stride2, int N, int H, int W, int C, int KN, int KH, int KW, float *dev_Y,
+               void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * The second half of tab_conv2d on an activation that is already packed (the output of
+ * tab_quantize with bitwidth 2 for TNN/TBN, 1 for BTN/BNN): zero padding, im2row and the
+ * popcount GEMM (PadKernel + Img2RowKernel + GEMMWithCuda, TAB_GEMM.cuh:22-115) fused in
+ * one kernel.  dev_QX int64 [N*H*W*PC*abits]; other arguments as in tab_conv2d.
+ */
+int tab_conv2d_packed(const int64_t *dev_QX, const int64_t *dev_QW, const int32_t *dev_btn,
+                      int type, int padding1, int padding2, int stride1, int stride2, int N,
+                      int H, int W, int C, int KN, int KH, int KW, float *dev_Y, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TAB_AMD_H */

@@ -1,0 +1,157 @@
+"""tab_amd - MI355X (gfx950) implementation of TAB's quantize + bitwise-conv operators.
+
+Host-side mirror of the reference's operator interface (TAB_GPU.cpp:34-65): the same two
+calls, positional argument lists, return tensors and error behaviour, on top of the C ABI
+in include/tab_amd.h.  PyTorch only supplies device memory and the current stream.
+
+    QW, BTN_W = Quantize(w, w_ths, bitwidth, KN, KH, KW, C)
+    y = Conv2d(x, QW, x_ths, BTN_W, type, pad1, pad2, stride1, stride2, N, H, W, C, KN, KH, KW)
+"""
+import torch
+
+from . import _capi
+
+_lib = _capi.load()
+TabError = _capi.TabError
+
+TNN, TBN, BTN, BNN = 0, 1, 2, 3
+
+
+def version():
+    return _lib.tab_version().decode()
+
+
+def _check_input(t, name):
+    # CHECK_INPUT of the reference (TAB_GPU.cpp:7-9): device + contiguity, as RuntimeError
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+
+
+def _check_dtype(t, dtype, name):
+    # The reference converts with .toType() on a temporary (TAB_GEMM.cu:279-280,341-347),
+    # which dangles when a conversion really happens; exact dtypes are required instead.
+    if t.dtype != dtype:
+        raise RuntimeError(f"{name} must have dtype {dtype}, got {t.dtype}")
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def packed_channels(C):
+    return _lib.tab_packed_channels(int(C))
+
+
+def out_shape(H, W, KH, KW, pad1, pad2, stride1, stride2):
+    """(OH, OW) by the reference's integer-division formula (TAB_GEMM.cu:354-357)."""
+    return (_lib.tab_out_extent(H, pad1, KH, stride1), _lib.tab_out_extent(W, pad2, KW, stride2))
+
+
+def Quantize(X, thresholds, bitwidth, N, H, W, C):
+    """Ternarize (bitwidth 2) or binarize (bitwidth 1) NHWC fp32 data and pack 64 channels
+    per int64 word.  Returns [QX, BTN]: QX int64 (N,H,W,PC,bitwidth), BTN int32 (N,)
+    (TAB_GPU.cpp:53-58, TAB_GEMM.cu:250-322)."""
+    _check_input(X, "X")
+    _check_input(thresholds, "thresholds")
+    _check_dtype(X, torch.float32, "X")
+    _check_dtype(thresholds, torch.float32, "thresholds")
+    bitwidth, N, H, W, C = int(bitwidth), int(N), int(H), int(W), int(C)
+    if bitwidth not in (1, 2):
+        raise RuntimeError(f"bitwidth must be 1 or 2, got {bitwidth}")
+    if min(N, H, W, C) < 1:
+        raise RuntimeError("N, H, W, C must be positive")
+    if X.numel() != N * H * W * C:
+        raise RuntimeError(f"X has {X.numel()} elements, expected N*H*W*C = {N * H * W * C}")
+    if thresholds.numel() < N:
+        raise RuntimeError(f"thresholds has {thresholds.numel()} elements, expected at least N = {N}")
+    if thresholds.device != X.device:
+        raise RuntimeError("X and thresholds must be on the same device")
+    PC = packed_channels(C)
+    with torch.cuda.device(X.device):
+        QX = torch.empty((N, H, W, PC, bitwidth), dtype=torch.int64, device=X.device)
+        BTN = torch.empty((N,), dtype=torch.int32, device=X.device)
+        _capi.check(_lib, _lib.tab_quantize(X.data_ptr(), thresholds.data_ptr(), bitwidth, N, H, W, C,
+                                            QX.data_ptr(), BTN.data_ptr(), _stream()))
+    return [QX, BTN]
+
+
+def _conv_checks(QW, btn, type, N, H, W, C, KN, KH, KW, pad1, pad2, stride1, stride2):
+    if type not in (0, 1, 2, 3):
+        raise RuntimeError(f"type must be 0 (TNN), 1 (TBN), 2 (BTN) or 3 (BNN), got {type}")
+    if min(N, H, W, C, KN, KH, KW) < 1 or min(pad1, pad2) < 0 or min(stride1, stride2) < 1:
+        raise RuntimeError("sizes must be positive, padding >= 0 and stride >= 1")
+    wbits = 2 if type in (0, 2) else 1
+    need = KN * KH * KW * packed_channels(C) * wbits
+    if QW.numel() != need:
+        raise RuntimeError(f"QW has {QW.numel()} words, type {type} expects KN*KH*KW*PC*{wbits} = {need}")
+    if type == 2 and btn.numel() < KN:
+        raise RuntimeError(f"btn has {btn.numel()} elements, expected at least KN = {KN}")
+    OH, OW = out_shape(H, W, KH, KW, pad1, pad2, stride1, stride2)
+    if OH < 1 or OW < 1:
+        raise RuntimeError(f"empty output: OH={OH}, OW={OW}")
+    return OH, OW
+
+
+def Conv2d(X, QW, thresholds, btn, type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW):
+    """Quantize the NHWC fp32 activation on the fly (ternary for types 0/1, binary for 2/3)
+    and convolve it with the packed weights by XOR/AND + popcount.  Returns fp32 shaped
+    (N,KN,OH,OW) whose memory is ordered (n,oh,ow,kn), exactly as the reference's reshape
+    of its GEMM result (TAB_GPU.cpp:34-42, TAB_GEMM.cu:325-527)."""
+    for t, name in ((X, "X"), (QW, "QW"), (thresholds, "thresholds"), (btn, "btn")):
+        _check_input(t, name)
+    _check_dtype(X, torch.float32, "X")
+    _check_dtype(QW, torch.int64, "QW")
+    _check_dtype(thresholds, torch.float32, "thresholds")
+    _check_dtype(btn, torch.int32, "btn")
+    (type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW) = (
+        int(v) for v in (type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW))
+    OH, OW = _conv_checks(QW, btn, type, N, H, W, C, KN, KH, KW, padding1, padding2, stride1, stride2)
+    if X.numel() != N * H * W * C:
+        raise RuntimeError(f"X has {X.numel()} elements, expected N*H*W*C = {N * H * W * C}")
+    if thresholds.numel() < N:
+        raise RuntimeError(f"thresholds has {thresholds.numel()} elements, expected at least N = {N}")
+    for t, name in ((QW, "QW"), (thresholds, "thresholds"), (btn, "btn")):
+        if t.device != X.device:
+            raise RuntimeError(f"X and {name} must be on the same device")
+    with torch.cuda.device(X.device):
+        Y = torch.empty((N, KN, OH, OW), dtype=torch.float32, device=X.device)
+        ws_bytes = _lib.tab_conv2d_workspace_bytes(type, N, H, W, C)
+        ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=X.device)
+        _capi.check(_lib, _lib.tab_conv2d(X.data_ptr(), QW.data_ptr(), thresholds.data_ptr(), btn.data_ptr(),
+                                          type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW,
+                                          Y.data_ptr(), ws.data_ptr(), ws_bytes, _stream()))
+    return Y
+
+
+def Conv2dPacked(QX, QW, btn, type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW):
+    """Conv2d on an activation already packed by Quantize (bitwidth 2 for types 0/1,
+    1 for types 2/3): the pad + im2row + GEMM stages of TAB_GEMM.cu:447-509 only."""
+    for t, name in ((QX, "QX"), (QW, "QW"), (btn, "btn")):
+        _check_input(t, name)
+    _check_dtype(QX, torch.int64, "QX")
+    _check_dtype(QW, torch.int64, "QW")
+    _check_dtype(btn, torch.int32, "btn")
+    (type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW) = (
+        int(v) for v in (type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW))
+    OH, OW = _conv_checks(QW, btn, type, N, H, W, C, KN, KH, KW, padding1, padding2, stride1, stride2)
+    abits = 2 if type < 2 else 1
+    if QX.numel() != N * H * W * packed_channels(C) * abits:
+        raise RuntimeError(f"QX has {QX.numel()} words, type {type} expects N*H*W*PC*{abits}")
+    with torch.cuda.device(QX.device):
+        Y = torch.empty((N, KN, OH, OW), dtype=torch.float32, device=QX.device)
+        _capi.check(_lib, _lib.tab_conv2d_packed(QX.data_ptr(), QW.data_ptr(), btn.data_ptr(), type,
+                                                 padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW,
+                                                 Y.data_ptr(), _stream()))
+    return Y
+
+
+# names of the reference's CPU module (TAB_CPU.cpp:636-639)
+TAB_Quantize = Quantize
+TAB_Conv2d = Conv2d
+
+__all__ = ["Quantize", "Conv2d", "Conv2dPacked", "TAB_Quantize", "TAB_Conv2d", "TabError",
+           "packed_channels", "out_shape", "version", "TNN", "TBN", "BTN", "BNN"]

@@ -1,0 +1,30 @@
+"""Build recipe of the HIP library: hipcc, gfx950 only, in-tree output (tab_amd/lib/)."""
+import os
+import subprocess
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB_DIR = os.path.join(HERE, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libtab_amd.so")
+SOURCES = ["tab_capi.hip", "tab_conv.hip", "tab_quantize.hip"]
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+# -packed-fp32-ops: keep the compiler from forming packed-FP32 VALU ops from float code.
+HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def build_library(verbose=False):
+    """Compile every HIP source and link libtab_amd.so. Always recompiles."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    cmd = [HIPCC] + HIP_FLAGS + ["-shared", "-o", LIB_PATH] + [os.path.join(CSRC, s) for s in SOURCES]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + out)
+    if verbose and out.strip():
+        print(out)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build_library(verbose=True))

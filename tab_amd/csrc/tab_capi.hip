@@ -1,0 +1,161 @@
+// C ABI of the library (declared in include/tab_amd.h): argument checks, workspace
+// carving and kernel launches.  No allocation, no synchronisation, no host<->device copy.
+#include "../../include/tab_amd.h"
+#include "tab_common.h"
+
+#include <cstdarg>
+#include <cstdio>
+
+namespace {
+
+thread_local char g_last_error[512] = "";
+
+int fail(int status, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+    va_end(ap);
+    return status;
+}
+
+int device_fail(hipError_t e, const char *what)
+{
+    return fail(TAB_ERR_DEVICE, "%s: %s", what, hipGetErrorString(e));
+}
+
+constexpr long kMaxIndex = 0x7fffffffL;  // kernels index rows/pixels with 32-bit ints
+
+struct ConvShape {
+    int PC, OH, OW, abits, wbits;
+    long M, G;
+};
+
+// Shared validation of the conv geometry (TAB_GEMM.cu:354-379).
+int check_conv(int type, int p1, int p2, int s1, int s2, int N, int H, int W, int C, int KN,
+               int KH, int KW, ConvShape *s)
+{
+    if (type < 0 || type > 3) return fail(TAB_ERR_BAD_ARGUMENT, "type must be 0 (TNN), 1 (TBN), 2 (BTN) or 3 (BNN), got %d", type);
+    if (N < 1 || H < 1 || W < 1 || C < 1 || KN < 1 || KH < 1 || KW < 1)
+        return fail(TAB_ERR_BAD_ARGUMENT, "N, H, W, C, KN, KH, KW must be positive");
+    if (p1 < 0 || p2 < 0 || s1 < 1 || s2 < 1)
+        return fail(TAB_ERR_BAD_ARGUMENT, "padding must be >= 0 and stride >= 1");
+    s->PC = tab_packed_channels(C);
+    s->OH = tab_out_extent(H, p1, KH, s1);
+    s->OW = tab_out_extent(W, p2, KW, s2);
+    if (s->OH < 1 || s->OW < 1)
+        return fail(TAB_ERR_BAD_SHAPE, "empty output: OH=%d OW=%d", s->OH, s->OW);
+    s->abits = (type < 2) ? 2 : 1;
+    s->wbits = (type == 0 || type == 2) ? 2 : 1;
+    s->M = (long)N * s->OH * s->OW;
+    s->G = (long)KH * KW * s->PC;
+    if (s->M > kMaxIndex || s->G >= 65536 || s->PC >= 65536 || KW >= 65536 ||
+        (long)N * H * W > kMaxIndex || (long)H * W * s->PC * 2 > kMaxIndex)
+        return fail(TAB_ERR_BAD_SHAPE, "problem too large for 32-bit row indices (M=%ld, K words=%ld)", s->M, s->G);
+    return TAB_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *tab_status_string(int status)
+{
+    switch (status) {
+    case TAB_OK: return "TAB_OK";
+    case TAB_ERR_BAD_ARGUMENT: return "TAB_ERR_BAD_ARGUMENT";
+    case TAB_ERR_BAD_SHAPE: return "TAB_ERR_BAD_SHAPE";
+    case TAB_ERR_WORKSPACE: return "TAB_ERR_WORKSPACE";
+    case TAB_ERR_DEVICE: return "TAB_ERR_DEVICE";
+    default: return "TAB_ERR_UNKNOWN";
+    }
+}
+
+const char *tab_last_error(void) { return g_last_error; }
+
+const char *tab_version(void) { return "tab_amd 0.1 gfx950"; }
+
+int tab_packed_channels(int C) { return (C + tab::kWordBits - 1) / tab::kWordBits; }
+
+int tab_out_extent(int in, int pad, int k, int stride)
+{
+    if (stride < 1) return 0;
+    return (in + 2 * pad - k + 1) / stride;
+}
+
+int tab_quantize(const float *dev_X, const float *dev_ths, int bitwidth, int N, int H, int W,
+                 int C, int64_t *dev_QX, int32_t *dev_BTN, void *stream)
+{
+    if (bitwidth != 1 && bitwidth != 2) return fail(TAB_ERR_BAD_ARGUMENT, "bitwidth must be 1 or 2, got %d", bitwidth);
+    if (N < 1 || H < 1 || W < 1 || C < 1) return fail(TAB_ERR_BAD_ARGUMENT, "N, H, W, C must be positive");
+    if (!dev_X || !dev_ths || !dev_QX || !dev_BTN) return fail(TAB_ERR_BAD_ARGUMENT, "null device pointer");
+    hipError_t e = tab::launch_quantize(dev_X, dev_ths, bitwidth, (long)H * W, N, C,
+                                        reinterpret_cast<uint64_t *>(dev_QX), dev_BTN,
+                                        static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return device_fail(e, "quantize launch");
+    return TAB_OK;
+}
+
+size_t tab_conv2d_workspace_bytes(int type, int N, int H, int W, int C)
+{
+    if (type < 0 || type > 3 || N < 1 || H < 1 || W < 1 || C < 1) return 0;
+    const size_t abits = (type < 2) ? 2 : 1;
+    return (size_t)N * H * W * tab_packed_channels(C) * abits * sizeof(int64_t);
+}
+
+int tab_conv2d_packed(const int64_t *dev_QX, const int64_t *dev_QW, const int32_t *dev_btn,
+                      int type, int padding1, int padding2, int stride1, int stride2, int N,
+                      int H, int W, int C, int KN, int KH, int KW, float *dev_Y, void *stream)
+{
+    ConvShape s;
+    int rc = check_conv(type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW, &s);
+    if (rc != TAB_OK) return rc;
+    if (!dev_QX || !dev_QW || !dev_Y) return fail(TAB_ERR_BAD_ARGUMENT, "null device pointer");
+    if (type == TAB_BTN && !dev_btn) return fail(TAB_ERR_BAD_ARGUMENT, "btn is required for type 2 (BTN)");
+    if (((uintptr_t)dev_QX % (8 * s.abits)) || ((uintptr_t)dev_QW % (8 * s.wbits)) || ((uintptr_t)dev_Y % 16))
+        return fail(TAB_ERR_BAD_ARGUMENT, "QX/QW must be aligned to a whole packed element and Y to 16 bytes");
+
+    tab::ConvArgs a;
+    a.qx = reinterpret_cast<const uint64_t *>(dev_QX);
+    a.qw = reinterpret_cast<const uint64_t *>(dev_QW);
+    a.btn = dev_btn;
+    a.y = dev_Y;
+    a.N = N; a.H = H; a.W = W; a.PC = s.PC;
+    a.KN = KN; a.KH = KH; a.KW = KW;
+    a.p1 = padding1; a.p2 = padding2; a.s1 = stride1; a.s2 = stride2;
+    a.OH = s.OH; a.OW = s.OW;
+    a.M = (int)s.M;
+    a.G = (int)s.G;
+    a.kcw = 0; a.nchunks = 0; a.tiles_m = 0;
+    a.num = KH * KW * C;
+    a.div_pc = tab::make_fastdiv((uint32_t)s.PC);
+    a.div_kw = tab::make_fastdiv((uint32_t)KW);
+    hipError_t e = tab::launch_conv(type, a, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return device_fail(e, "conv launch");
+    return TAB_OK;
+}
+
+int tab_conv2d(const float *dev_X, const int64_t *dev_QW, const float *dev_ths,
+               const int32_t *dev_btn, int type, int padding1, int padding2, int stride1,
+               int stride2, int N, int H, int W, int C, int KN, int KH, int KW, float *dev_Y,
+               void *workspace, size_t workspace_bytes, void *stream)
+{
+    ConvShape s;
+    int rc = check_conv(type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW, &s);
+    if (rc != TAB_OK) return rc;
+    if (!dev_X || !dev_ths) return fail(TAB_ERR_BAD_ARGUMENT, "null device pointer");
+    const size_t need = tab_conv2d_workspace_bytes(type, N, H, W, C);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace % 16))
+        return fail(TAB_ERR_WORKSPACE, "workspace must be 16-byte aligned and hold %zu bytes (got %zu)", need, workspace_bytes);
+    // stage 1: quantize + pack the activation (TAB_GEMM.cu:419-426); no btn for activations
+    hipError_t e = tab::launch_quantize(dev_X, dev_ths, s.abits, (long)H * W, N, C,
+                                        reinterpret_cast<uint64_t *>(workspace), nullptr,
+                                        static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return device_fail(e, "quantize launch");
+    // stage 2: pad + im2row + GEMM, fused
+    return tab_conv2d_packed(reinterpret_cast<const int64_t *>(workspace), dev_QW, dev_btn, type,
+                             padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW, dev_Y,
+                             stream);
+}
+
+}  // extern "C"

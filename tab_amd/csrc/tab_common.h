@@ -1,0 +1,55 @@
+// Shared declarations of the gfx950 TAB kernels (internal; the public surface is
+// include/tab_amd.h).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace tab {
+
+constexpr int kWordBits = 64;  // channels per packed int64 word (CNTBITS, TAB_GEMM.cuh:10)
+
+// Exact x / d for x < 65536 and 1 <= d < 65536 with one multiply-high:
+// magic = floor(2^32 / d) + 1 gives floor(x * magic / 2^32) == floor(x / d) whenever
+// x * d < 2^32.  d == 1 has no 32-bit magic and is passed through.
+struct FastDiv {
+    uint32_t magic;
+    uint32_t d;
+};
+inline FastDiv make_fastdiv(uint32_t d)
+{
+    FastDiv f;
+    f.d = d;
+    f.magic = d > 1 ? (uint32_t)(0x100000000ull / d) + 1u : 0u;
+    return f;
+}
+__device__ __forceinline__ uint32_t fastdiv(uint32_t x, FastDiv f)
+{
+    return f.d == 1 ? x : __umulhi(x, f.magic);
+}
+
+// Arguments of the fused pad + im2row + popcount-GEMM kernel.
+struct ConvArgs {
+    const uint64_t *qx;  // packed activation [N][H][W][PC][APL]
+    const uint64_t *qw;  // packed weight     [KN][KH][KW][PC][BPL]
+    const int32_t *btn;  // [KN] (BTN only)
+    float *y;            // [M][KN]
+    int N, H, W, PC;
+    int KN, KH, KW;
+    int p1, p2, s1, s2;
+    int OH, OW;
+    int M;         // N*OH*OW
+    int G;         // KH*KW*PC, packed words along K per plane
+    int kcw;       // words per K chunk (<= kMaxChunkWords)
+    int nchunks;   // ceil(G / kcw)
+    int num;       // KH*KW*C (BNN constant)
+    int tiles_m;   // ceil(M / BM)
+    FastDiv div_pc, div_kw;
+};
+
+// Launchers (tab_conv.hip / tab_quantize.hip); they enqueue on `stream` and return the
+// launch status.
+hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream);
+hipError_t launch_quantize(const float *x, const float *ths, int bitwidth, long pixels_per_item,
+                           long items, int C, uint64_t *qx, int32_t *btn, hipStream_t stream);
+
+}  // namespace tab

@@ -1,0 +1,316 @@
+// Fused zero-pad + im2row + popcount GEMM for gfx950 (wave64), all four TAB types.
+//
+// Replaces PadKernel + Img2RowKernel (TAB_GEMM.cuh:73-115) and TNNGEMM/TBNGEMM/BTNGEMM/
+// BNNGEMM (TAB_GEMM.cu:25-147): Y[m][kn] = f(sum over k of popcount(op(A[m][k], B[kn][k])))
+// with A the im2row view of the packed activation, never materialised: padding and stride
+// live in the address math, out-of-range taps read all-zero words (TAB_CPU.cpp:39,155).
+//
+// Work decomposition: a 256-thread workgroup owns a BM x BN tile of Y (BM = 16*TM output
+// pixels, BN = 64*NG filters); thread (ty, tx) of the 16x16 grid owns rows ty*TM.. and the
+// column quads g*64 + tx*4.. .  K is walked in chunks of `kcw` packed 64-bit words; each
+// chunk of both operands is staged in LDS, split into 32-bit halves and stored k-major
+// ([plane][q][row], q = 2*word + half) so that a thread fetches its TM rows / 4 columns of
+// one k-slice with 128-bit LDS reads (A reads broadcast over the 16 tx lanes, B reads are
+// 256 B contiguous per 16 lanes).  The inner loop is pure VALU: XOR/AND + v_bcnt_u32_b32
+// with the count accumulated in the instruction's addend.
+#include "tab_common.h"
+
+namespace tab {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kMaxChunkWords = 8;             // packed 64-bit words of K per chunk, at most
+constexpr int kMaxQ = 2 * kMaxChunkWords;     // 32-bit k-slices per chunk
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <int TYPE> struct Planes {
+    static constexpr int A = (TYPE == 0 || TYPE == 1) ? 2 : 1;  // activation planes (TAB_GEMM.cu:367-372)
+    static constexpr int B = (TYPE == 0 || TYPE == 2) ? 2 : 1;  // weight planes (TAB_GEMM.cu:374-379)
+};
+
+// Fetch of one packed word (all planes) of one row of an operand, kept in registers
+// between the global load and the LDS store.
+template <int PL> struct Item {
+    uint32_t d[2 * PL];  // plane-major in memory: [plane][half] as 64-bit words
+};
+
+template <int PL>
+__device__ __forceinline__ Item<PL> load_item(const uint64_t *p, bool valid)
+{
+    Item<PL> it;
+    if (PL == 2) {
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (valid) v = *reinterpret_cast<const u32x4 *>(p);
+        it.d[0] = v[0]; it.d[1] = v[1]; it.d[2] = v[2]; it.d[3] = v[3];
+    } else {
+        u32x2 v = {0u, 0u};
+        if (valid) v = *reinterpret_cast<const u32x2 *>(p);
+        it.d[0] = v[0]; it.d[1] = v[1];
+    }
+    return it;
+}
+
+// LDS placement: dword index ((plane*kMaxQ + q) * ROWS + row)
+template <int PL, int ROWS>
+__device__ __forceinline__ void store_item(uint32_t *lds, const Item<PL> &it, int word, int row)
+{
+#pragma unroll
+    for (int pl = 0; pl < PL; pl++)
+#pragma unroll
+        for (int half = 0; half < 2; half++)
+            lds[((pl * kMaxQ) + 2 * word + half) * ROWS + row] = it.d[pl * 2 + half];
+}
+
+template <int TYPE, int TM, int NG>
+__global__ __launch_bounds__(kThreads) void conv_popcount(const ConvArgs p)
+{
+    constexpr int APL = Planes<TYPE>::A, BPL = Planes<TYPE>::B;
+    constexpr int BM = 16 * TM, BN = 64 * NG, TN = 4 * NG;
+    constexpr int A_DWORDS = APL * kMaxQ * BM, B_DWORDS = BPL * kMaxQ * BN;
+    constexpr int A_STEP = kThreads / BM;                      // words fetched per pass over the tile rows
+    constexpr int B_STEP = kThreads / BN;
+    constexpr int A_ITEMS = (kMaxChunkWords + A_STEP - 1) / A_STEP;
+    constexpr int B_ITEMS = (kMaxChunkWords + B_STEP - 1) / B_STEP;
+    static_assert(kThreads % BM == 0 && kThreads % BN == 0, "tile rows must divide the workgroup");
+    static_assert(TM % 4 == 0 || TM == 2, "TM is read with 64- or 128-bit LDS loads");
+
+    __shared__ __attribute__((aligned(16))) uint32_t lds[2][A_DWORDS + B_DWORDS];
+
+    const int tid = threadIdx.x;
+    const int tx = tid & 15, ty = tid >> 4;
+    // consecutive workgroups walk M first so neighbours share the weight tile in L2
+    const int tile_m = blockIdx.x % p.tiles_m, tile_n = blockIdx.x / p.tiles_m;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    // ---- staging roles -------------------------------------------------------------------
+    // A: thread fetches words (a_w0 + i*A_STEP) of output pixel m0 + a_row
+    const int a_row = tid % BM, a_w0 = tid / BM;
+    const int a_m = m0 + a_row;
+    const bool a_live = a_m < p.M;
+    int ih0, iw0;
+    const uint64_t *a_img;
+    {
+        const int mm = a_live ? a_m : 0;
+        const int n = mm / (p.OH * p.OW);
+        const int r = mm - n * (p.OH * p.OW);
+        const int oh = r / p.OW, ow = r - oh * p.OW;
+        ih0 = oh * p.s1 - p.p1;
+        iw0 = ow * p.s2 - p.p2;
+        a_img = p.qx + (size_t)n * p.H * p.W * p.PC * APL;
+    }
+    // B: thread fetches words (b_w0 + i*B_STEP) of filter n0 + b_row
+    const int b_row = tid % BN, b_w0 = tid / BN;
+    const bool b_live = (n0 + b_row) < p.KN;
+    const uint64_t *b_flt = p.qw + (size_t)(b_live ? n0 + b_row : 0) * p.G * BPL;
+
+    Item<APL> a_reg[A_ITEMS];
+    Item<BPL> b_reg[B_ITEMS];
+
+    auto fetch = [&](int chunk) {
+        const int g0 = chunk * p.kcw;
+#pragma unroll
+        for (int i = 0; i < A_ITEMS; i++) {
+            const int w = a_w0 + i * A_STEP;
+            const int g = g0 + w;
+            // g is uniform over the wave when BM >= 64; the tap decode is a few multiplies
+            const uint32_t tap = fastdiv((uint32_t)g, p.div_pc);
+            const int pc = g - (int)tap * p.PC;
+            const uint32_t kh = fastdiv(tap, p.div_kw);
+            const int kw = (int)tap - (int)kh * p.KW;
+            const int ih = ih0 + (int)kh, iw = iw0 + kw;
+            const bool ok = a_live && w < p.kcw && g < p.G && (unsigned)ih < (unsigned)p.H &&
+                            (unsigned)iw < (unsigned)p.W;
+            const size_t off = ok ? ((size_t)(ih * p.W + iw) * p.PC + pc) * APL : 0;
+            a_reg[i] = load_item<APL>(a_img + off, ok);
+        }
+#pragma unroll
+        for (int i = 0; i < B_ITEMS; i++) {
+            const int w = b_w0 + i * B_STEP;
+            const int g = g0 + w;
+            const bool ok = b_live && w < p.kcw && g < p.G;
+            b_reg[i] = load_item<BPL>(b_flt + (ok ? (size_t)g * BPL : 0), ok);
+        }
+    };
+    auto stage = [&](int buf) {
+        uint32_t *la = lds[buf], *lb = lds[buf] + A_DWORDS;
+#pragma unroll
+        for (int i = 0; i < A_ITEMS; i++) {
+            const int w = a_w0 + i * A_STEP;
+            if (w < kMaxChunkWords) store_item<APL, BM>(la, a_reg[i], w, a_row);
+        }
+#pragma unroll
+        for (int i = 0; i < B_ITEMS; i++) {
+            const int w = b_w0 + i * B_STEP;
+            if (w < kMaxChunkWords) store_item<BPL, BN>(lb, b_reg[i], w, b_row);
+        }
+    };
+
+    // ---- accumulators --------------------------------------------------------------------
+    // acc: popcount of the "negative" word (TNN/TBN/BTN) or of a^b (BNN);
+    // nzc: TNN popcount(a1 & b1) per output; TBN popcount(a1) per row (independent of kn).
+    int acc[TM][TN];
+    int nzc[TYPE == 0 ? TM : 1][TYPE == 0 ? TN : 1];
+    int row_nz[TYPE == 1 ? TM : 1];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            acc[i][j] = 0;
+            if (TYPE == 0) nzc[i][j] = 0;
+        }
+    if (TYPE == 1) {
+#pragma unroll
+        for (int i = 0; i < TM; i++) row_nz[i] = 0;
+    }
+
+    fetch(0);
+    stage(0);
+    __syncthreads();
+
+    for (int chunk = 0; chunk < p.nchunks; chunk++) {
+        const bool more = chunk + 1 < p.nchunks;
+        if (more) fetch(chunk + 1);
+
+        const uint32_t *la = lds[chunk & 1], *lb = lds[chunk & 1] + A_DWORDS;
+        const int words_here = (p.G - chunk * p.kcw < p.kcw) ? p.G - chunk * p.kcw : p.kcw;
+        const int nq = 2 * words_here;
+        for (int q = 0; q < nq; q++) {
+            uint32_t a[APL][TM], b[BPL][TN];
+#pragma unroll
+            for (int pl = 0; pl < APL; pl++) {
+                const uint32_t *src = la + (pl * kMaxQ + q) * BM + ty * TM;
+                if (TM == 2) {
+                    const u32x2 v = *reinterpret_cast<const u32x2 *>(src);
+                    a[pl][0] = v[0]; a[pl][1] = v[1];
+                } else {
+#pragma unroll
+                    for (int i4 = 0; i4 < TM / 4; i4++) {
+                        const u32x4 v = *reinterpret_cast<const u32x4 *>(src + 4 * i4);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) a[pl][4 * i4 + e] = v[e];
+                    }
+                }
+            }
+#pragma unroll
+            for (int pl = 0; pl < BPL; pl++)
+#pragma unroll
+                for (int g = 0; g < NG; g++) {
+                    const u32x4 v = *reinterpret_cast<const u32x4 *>(lb + (pl * kMaxQ + q) * BN + g * 64 + tx * 4);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) b[pl][4 * g + e] = v[e];
+                }
+
+            if (TYPE == 1) {
+#pragma unroll
+                for (int i = 0; i < TM; i++) row_nz[i] += __builtin_popcount(a[APL - 1][i]);
+            }
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    if (TYPE == 0) {
+                        // TAB_GEMM.cu:48-51
+                        const uint32_t both = a[1][i] & b[1][j];
+                        nzc[i][j] += __builtin_popcount(both);
+                        acc[i][j] += __builtin_popcount((a[0][i] ^ b[0][j]) & both);
+                    } else if (TYPE == 1) {
+                        // TAB_GEMM.cu:81-84; popcount(a1) is summed once per row above
+                        acc[i][j] += __builtin_popcount((a[0][i] ^ b[0][j]) & a[1][i]);
+                    } else if (TYPE == 2) {
+                        // TAB_GEMM.cu:113-114
+                        acc[i][j] += __builtin_popcount((a[0][i] ^ b[0][j]) & b[1][j]);
+                    } else {
+                        // TAB_GEMM.cu:142
+                        acc[i][j] += __builtin_popcount(a[0][i] ^ b[0][j]);
+                    }
+                }
+        }
+
+        if (more) stage((chunk + 1) & 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: integer result -> fp32, Y[m*KN + kn] (TAB_GEMM.cu:53,86,116,144) --------
+    const bool vec_ok = (p.KN & 3) == 0;
+#pragma unroll
+    for (int g = 0; g < NG; g++) {
+        const int kn = n0 + g * 64 + tx * 4;
+        int bias[4] = {0, 0, 0, 0};
+        if (TYPE == 2) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) bias[e] = (kn + e < p.KN) ? p.btn[kn + e] : 0;
+        }
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            const int m = m0 + ty * TM + i;
+            if (m >= p.M) continue;
+            float out[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int j = 4 * g + e;
+                int v;
+                if (TYPE == 0) v = nzc[i][j] - 2 * acc[i][j];
+                else if (TYPE == 1) v = row_nz[i] - 2 * acc[i][j];
+                else if (TYPE == 2) v = bias[e] - 2 * acc[i][j];
+                else v = p.num - 2 * acc[i][j];
+                out[e] = (float)v;
+            }
+            float *dst = p.y + (size_t)m * p.KN + kn;
+            if (vec_ok && kn + 3 < p.KN) {
+                *reinterpret_cast<f32x4 *>(dst) = f32x4{out[0], out[1], out[2], out[3]};
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (kn + e < p.KN) dst[e] = out[e];
+            }
+        }
+    }
+}
+
+template <int TYPE, int TM, int NG>
+hipError_t launch_tile(ConvArgs a, hipStream_t stream)
+{
+    constexpr int BM = 16 * TM, BN = 64 * NG;
+    a.tiles_m = (a.M + BM - 1) / BM;
+    const long tiles_n = (a.KN + BN - 1) / BN;
+    const long blocks = (long)a.tiles_m * tiles_n;
+    if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
+    conv_popcount<TYPE, TM, NG><<<dim3((unsigned)blocks), dim3(kThreads), 0, stream>>>(a);
+    return hipGetLastError();
+}
+
+// Tile choice: the largest tile that still gives every CU a few workgroups; small layers
+// fall back to smaller tiles so that the 256 CUs are not left idle.
+template <int TYPE>
+hipError_t launch_type(const ConvArgs &a, hipStream_t stream)
+{
+    const long want = 2 * 256;  // at least two workgroups per CU
+    auto tiles = [&](int bm, int bn) { return (long)((a.M + bm - 1) / bm) * ((a.KN + bn - 1) / bn); };
+    if (TYPE != 0 && a.KN > 64 && tiles(128, 128) >= want) return launch_tile<TYPE, 8, (TYPE == 0 ? 1 : 2)>(a, stream);
+    if (tiles(128, 64) >= want) return launch_tile<TYPE, 8, 1>(a, stream);
+    if (tiles(64, 64) >= want) return launch_tile<TYPE, 4, 1>(a, stream);
+    return launch_tile<TYPE, 2, 1>(a, stream);
+}
+
+}  // namespace
+
+hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream)
+{
+    ConvArgs a = args;
+    // chunk length: at most kMaxChunkWords, and such that the chunks are of equal length
+    a.nchunks = (a.G + kMaxChunkWords - 1) / kMaxChunkWords;
+    a.kcw = (a.G + a.nchunks - 1) / a.nchunks;
+    a.nchunks = (a.G + a.kcw - 1) / a.kcw;
+    switch (type) {
+    case 0: return launch_type<0>(a, stream);
+    case 1: return launch_type<1>(a, stream);
+    case 2: return launch_type<2>(a, stream);
+    case 3: return launch_type<3>(a, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace tab

@@ -1,0 +1,220 @@
+// Quantizer / bit-packer for gfx950 (wave64): fp32 NHWC -> packed int64 bit planes.
+//
+// Semantics follow the reference kernels TerOnlyKernel (TAB_GEMM.cu:163-208) and
+// BinOnlyKernel (TAB_GEMM.cu:211-247) with the per-item threshold ths[n] of the CPU path
+// (TAB_CPU.cpp:67,72), plus BTN_Weight (TAB_GEMM.cu:150-160) for every item.
+//
+// The tensor is a sequence of "rows" of 64 consecutive channels; row r becomes packed
+// word r (C % 64 == 0) so the whole op is one streaming pass: 256 B in, 8 or 16 B out.
+#include "tab_common.h"
+
+namespace tab {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWavesPerBlock = kThreads / 64;
+constexpr int kLoadsPerLane = 8;                // float4 loads in flight per lane
+constexpr int kRowsPerWave = 4 * kLoadsPerLane; // each wave-wide float4 load covers 4 rows
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// OR over the 8 lanes of each half of a 16-lane DPP row; every lane gets the result.
+__device__ __forceinline__ uint32_t or_reduce8(uint32_t v)
+{
+    v |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]
+    v |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
+    v |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xF, 0xF, true);  // row_half_mirror
+    return v;
+}
+
+__device__ __forceinline__ int wave_sum(int v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+    return v;
+}
+
+// Compare one float4 against the threshold; bit e of the result belongs to element e.
+// Ternary: first test v > t (+1), only then v < -t (-1); both are strict and ordered, so
+// ties and NaN give 0 (TAB_GEMM.cu:184-192).  Binary: bit = v < t (TAB_GEMM.cu:231).
+template <int BITS>
+__device__ __forceinline__ void compare4(const floatx4 v, const float t, uint32_t &sign, uint32_t &nz)
+{
+    const float e[4] = {v[0], v[1], v[2], v[3]};
+    sign = 0;
+    nz = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        if (BITS == 2) {
+            const bool pos = e[i] > t;
+            const bool neg = !pos && (e[i] < -t);
+            nz |= (uint32_t)(pos || neg) << i;
+            sign |= (uint32_t)neg << i;
+        } else {
+            sign |= (uint32_t)(e[i] < t) << i;
+        }
+    }
+}
+
+// Fast path, C % 64 == 0 and X 16-byte aligned.
+// Lane layout: a 16-lane DPP row reads one 64-channel row as 16 float4 (256 B contiguous),
+// a wave reads 4 consecutive rows per load (1 KB contiguous) and keeps kLoadsPerLane loads
+// in flight.  Each lane turns its 4 compares into a nibble placed at bit 4*(lane%8); an OR
+// over 8 lanes yields the low (lanes 0-7) or high (lanes 8-15) 32 bits of the word.
+template <int BITS, bool WITH_BTN>
+__global__ __launch_bounds__(kThreads) void quantize_rows64(const floatx4 *__restrict__ x,
+                                                            const float *__restrict__ ths,
+                                                            uint32_t *__restrict__ q,
+                                                            int32_t *__restrict__ btn, long rows,
+                                                            long rows_per_item)
+{
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int sub = lane >> 4;  // which of the 4 rows of a load
+    const int l = lane & 15;    // float4 within the row
+    const long row0 = ((long)blockIdx.x * kWavesPerBlock + wave) * kRowsPerWave;
+    if (row0 >= rows) return;
+    const long row_last = (row0 + kRowsPerWave - 1 < rows ? row0 + kRowsPerWave - 1 : rows - 1);
+
+    floatx4 v[kLoadsPerLane];
+#pragma unroll
+    for (int u = 0; u < kLoadsPerLane; u++) {
+        const long r = row0 + u * 4 + sub;
+        v[u] = (r < rows) ? __builtin_nontemporal_load(&x[r * 16 + l]) : floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    const long item_first = row0 / rows_per_item;
+    const bool one_item = (row_last / rows_per_item) == item_first;  // wave-uniform
+    const float t_first = ths[item_first];
+    int count = 0;
+
+#pragma unroll
+    for (int u = 0; u < kLoadsPerLane; u++) {
+        const long r = row0 + u * 4 + sub;
+        float t = t_first;
+        long item = item_first;
+        if (!one_item) {
+            item = (r < rows ? r : rows - 1) / rows_per_item;
+            t = ths[item];
+        }
+        uint32_t sign, nz;
+        compare4<BITS>(v[u], t, sign, nz);
+        const int shift = 4 * (l & 7);
+        const uint32_t sign_word = or_reduce8(sign << shift);
+        if (BITS == 2) {
+            const uint32_t nz_word = or_reduce8(nz << shift);
+            if (WITH_BTN) {
+                if (one_item) {
+                    count += __builtin_popcount(nz);
+                } else if (r < rows && nz) {
+                    atomicAdd(&btn[item], __builtin_popcount(nz));
+                }
+            }
+            // dword (r*2 + plane)*2 + half; lanes 0/1 of each half-row store plane 0/1
+            if (r < rows && (l & 7) < 2) {
+                const int plane = l & 1, half = l >> 3;
+                q[(r * 2 + plane) * 2 + half] = plane ? nz_word : sign_word;
+            }
+        } else {
+            if (r < rows && (l & 7) == 0) q[r * 2 + (l >> 3)] = sign_word;
+        }
+    }
+    if (BITS == 2 && WITH_BTN && one_item) {
+        count = wave_sum(count);
+        if (lane == 0 && count) atomicAdd(&btn[item_first], count);
+    }
+}
+
+// General path (any C, any alignment): one wave per (pixel, word); lane i tests channel
+// word*64 + i and the two wave-wide ballots are the packed words, LSB first
+// (onebit[i] = 1 << i, TAB_GEMM.cu:252-258).  Unused high bits of a tail word stay 0
+// (TAB_GEMM.cu:203-206).
+template <int BITS, bool WITH_BTN>
+__global__ __launch_bounds__(kThreads) void quantize_ballot(const float *__restrict__ x,
+                                                            const float *__restrict__ ths,
+                                                            uint64_t *__restrict__ q,
+                                                            int32_t *__restrict__ btn, long pixels,
+                                                            long pixels_per_item, int C, int PC)
+{
+    const int lane = threadIdx.x & 63;
+    const long nwaves = (long)gridDim.x * kWavesPerBlock;
+    const long units = pixels * PC;
+    for (long unit = (long)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6); unit < units; unit += nwaves) {
+        const long pixel = unit / PC;
+        const int word = (int)(unit - pixel * PC);
+        const long item = pixel / pixels_per_item;
+        const float t = ths[item];
+        const int c = word * kWordBits + lane;
+        const bool live = c < C;
+        const float v = live ? x[pixel * C + c] : 0.f;
+        if (BITS == 2) {
+            const bool pos = live && (v > t);
+            const bool neg = live && !pos && (v < -t);
+            const uint64_t nz = __ballot(pos || neg);
+            const uint64_t sign = __ballot(neg);
+            if (lane == 0) {
+                q[unit * 2 + 0] = sign;
+                q[unit * 2 + 1] = nz;
+                if (WITH_BTN && nz) atomicAdd(&btn[item], __popcll(nz));
+            }
+        } else {
+            const uint64_t neg = __ballot(live && (v < t));
+            if (lane == 0) q[unit] = neg;
+        }
+    }
+}
+
+__global__ void fill_zero_i32(int32_t *p, long n)
+{
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+}  // namespace
+
+// x: fp32 [items][pixels_per_item][C]; qx: [items*pixels_per_item][PC][bitwidth];
+// btn: [items] or nullptr (then no counts are produced).
+hipError_t launch_quantize(const float *x, const float *ths, int bitwidth, long pixels_per_item,
+                           long items, int C, uint64_t *qx, int32_t *btn, hipStream_t stream)
+{
+    const int PC = (C + kWordBits - 1) / kWordBits;
+    const long pixels = items * pixels_per_item;
+    if (btn) {
+        // zero with a kernel, not a memset node, so callers may capture the call in a graph
+        fill_zero_i32<<<dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream>>>(btn, items);
+    }
+    const bool want_btn = btn != nullptr && bitwidth == 2;
+    const bool fast = (C % kWordBits == 0) && ((uintptr_t)x % 16 == 0);
+    if (fast) {
+        const long rows = pixels * PC;
+        const long rows_per_item = pixels_per_item * PC;
+        const long blocks = (rows + kRowsPerWave * kWavesPerBlock - 1) / (kRowsPerWave * kWavesPerBlock);
+        const dim3 grid((unsigned)blocks), block(kThreads);
+        const floatx4 *x4 = reinterpret_cast<const floatx4 *>(x);
+        uint32_t *q32 = reinterpret_cast<uint32_t *>(qx);
+        if (bitwidth == 2) {
+            if (want_btn)
+                quantize_rows64<2, true><<<grid, block, 0, stream>>>(x4, ths, q32, btn, rows, rows_per_item);
+            else
+                quantize_rows64<2, false><<<grid, block, 0, stream>>>(x4, ths, q32, btn, rows, rows_per_item);
+        } else {
+            quantize_rows64<1, false><<<grid, block, 0, stream>>>(x4, ths, q32, btn, rows, rows_per_item);
+        }
+    } else {
+        const long units = pixels * PC;
+        long blocks = (units + kWavesPerBlock - 1) / kWavesPerBlock;
+        if (blocks > 256 * 32) blocks = 256 * 32;  // grid-stride beyond 32 blocks per CU
+        const dim3 grid((unsigned)blocks), block(kThreads);
+        if (bitwidth == 2) {
+            if (want_btn)
+                quantize_ballot<2, true><<<grid, block, 0, stream>>>(x, ths, qx, btn, pixels, pixels_per_item, C, PC);
+            else
+                quantize_ballot<2, false><<<grid, block, 0, stream>>>(x, ths, qx, btn, pixels, pixels_per_item, C, PC);
+        } else {
+            quantize_ballot<1, false><<<grid, block, 0, stream>>>(x, ths, qx, btn, pixels, pixels_per_item, C, PC);
+        }
+    }
+    return hipGetLastError();
+}
+
+}  // namespace tab

@@ -1,0 +1,89 @@
+"""CPU-side checks of the boundary: the shared library loads, exports every symbol that
+include/tab_amd.h declares, its host-only entry points answer, and both the C ABI and the
+Python mirror reject bad arguments before anything is launched (no GPU is touched)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import tab_amd
+from tab_amd import _capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "tab_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tab_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_symbols()
+    assert {"tab_quantize", "tab_conv2d", "tab_conv2d_packed", "tab_conv2d_workspace_bytes"} <= set(names)
+    lib = ctypes.CDLL(_capi.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/tab_amd.h but not exported"
+    assert sorted(_capi.SIGNATURES) == names
+
+
+def test_host_only_entry_points():
+    lib = _capi.load()
+    assert lib.tab_version().decode().endswith("gfx950")
+    assert [lib.tab_packed_channels(c) for c in (1, 63, 64, 65, 256)] == [1, 1, 1, 2, 4]
+    # (in + 2*pad - k + 1) / stride, integer division (TAB_GEMM.cu:354-357)
+    assert lib.tab_out_extent(7, 1, 3, 2) == 3
+    assert lib.tab_out_extent(56, 1, 3, 2) == 28
+    assert lib.tab_out_extent(28, 1, 1, 2) == 15
+    assert lib.tab_status_string(0) == b"TAB_OK"
+    assert lib.tab_status_string(-3) == b"TAB_ERR_WORKSPACE"
+    # activation scratch: N*H*W*PC*abits int64 words
+    assert lib.tab_conv2d_workspace_bytes(0, 2, 5, 5, 70) == 2 * 5 * 5 * 2 * 2 * 8
+    assert lib.tab_conv2d_workspace_bytes(3, 2, 5, 5, 70) == 2 * 5 * 5 * 2 * 1 * 8
+    assert lib.tab_conv2d_workspace_bytes(4, 2, 5, 5, 70) == 0
+
+
+def test_c_abi_rejects_bad_arguments_without_launching():
+    lib = _capi.load()
+    p = 4096  # never dereferenced: every call below fails validation first
+    assert lib.tab_quantize(p, p, 3, 1, 1, 1, 64, p, p, None) == -1
+    assert b"bitwidth" in lib.tab_last_error()
+    assert lib.tab_quantize(None, p, 2, 1, 1, 1, 64, p, p, None) == -1
+    assert lib.tab_quantize(p, p, 2, 0, 1, 1, 64, p, p, None) == -1
+    conv = lambda **kw: lib.tab_conv2d(  # noqa: E731
+        kw.get("x", p), p, p, p, kw.get("type", 0), kw.get("p1", 1), 1, kw.get("s1", 1), 1,
+        1, kw.get("H", 8), 8, 64, 4, 3, 3, p, kw.get("ws", p), kw.get("ws_bytes", 1 << 20), None)
+    assert conv(type=4) == -1
+    assert conv(s1=0) == -1
+    assert conv(p1=-1) == -1
+    assert conv(H=1, p1=0) == -2 and b"empty output" in lib.tab_last_error()
+    assert conv(ws=None) == -3
+    assert conv(ws_bytes=8) == -3 and b"workspace" in lib.tab_last_error()
+    assert conv(x=None) == -1
+    # BTN needs btn
+    assert lib.tab_conv2d_packed(p, p, None, 2, 1, 1, 1, 1, 1, 8, 8, 64, 4, 3, 3, p, None) == -1
+    with pytest.raises(_capi.TabError, match="TAB_ERR_BAD_ARGUMENT"):
+        _capi.check(lib, lib.tab_quantize(p, p, 0, 1, 1, 1, 64, p, p, None))
+
+
+def test_python_mirror_names_and_input_checks():
+    # exported names of the CUDA module (TAB_GPU.cpp:62-65) and of the CPU module (TAB_CPU.cpp:636-639)
+    for name in ("Quantize", "Conv2d", "TAB_Quantize", "TAB_Conv2d"):
+        assert callable(getattr(tab_amd, name))
+    x = torch.zeros(1, 4, 4, 64)
+    ths = torch.zeros(1)
+    # CHECK_INPUT (TAB_GPU.cpp:7-9): a CPU tensor is refused with the reference's message
+    with pytest.raises(RuntimeError, match="X must be a CUDA tensor"):
+        tab_amd.Quantize(x, ths, 2, 1, 4, 4, 64)
+    with pytest.raises(RuntimeError, match="X must be a CUDA tensor"):
+        tab_amd.Conv2d(x, torch.zeros(4, dtype=torch.int64), ths, torch.zeros(4, dtype=torch.int32),
+                       0, 1, 1, 1, 1, 1, 4, 4, 64, 4, 3, 3)
+    assert tab_amd.out_shape(112, 112, 3, 3, 1, 1, 1, 1) == (112, 112)
+    assert tab_amd.packed_channels(256) == 4
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    with pytest.raises(ImportError, match="no fallback"):
+        _capi.load(str(tmp_path / "libtab_amd.so"))

@@ -1,0 +1,155 @@
+"""GPU parity of Conv2d / Conv2dPacked (through the C ABI) against the CPU oracle.
+Integer-valued results stored as fp32: the bar is bit-exact equality."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import tab_amd
+from helpers import TYPE_NAMES, act_bits, make_layer, weight_bits
+
+pytestmark = pytest.mark.gpu
+
+
+def _conv_case(type, N, H, W, C, KN, KH, KW, p1, p2, s1, s2, seed=0, relu=False):
+    print(f"[case] Conv2d {TYPE_NAMES[type]} N={N} {H}x{W}x{C}->{KN} k{KH}x{KW} pad({p1},{p2}) "
+          f"stride({s1},{s2}) relu={relu}", flush=True)
+    x, x_ths, w, w_ths = make_layer(type, N, H, W, C, KN, KH, KW, seed=seed, relu=relu)
+    qw_o, btn_o = oracle.quantize(w.numpy(), w_ths.numpy(), weight_bits(type), KN, KH, KW, C)
+    want = oracle.conv2d(x.numpy(), qw_o, x_ths.numpy(), btn_o, type, p1, p2, s1, s2, N, H, W, C, KN, KH, KW)
+
+    QW, BTN = tab_amd.Quantize(w.cuda(), w_ths.cuda(), weight_bits(type), KN, KH, KW, C)
+    y = tab_amd.Conv2d(x.cuda(), QW, x_ths.cuda(), BTN, type, p1, p2, s1, s2, N, H, W, C, KN, KH, KW)
+    torch.cuda.synchronize()
+    assert y.dtype == torch.float32 and tuple(y.shape) == want.shape
+    assert np.array_equal(QW.cpu().numpy(), qw_o) and np.array_equal(BTN.cpu().numpy(), btn_o)
+    got = y.cpu().numpy()
+    assert np.array_equal(got, want), f"max |diff| = {np.abs(got - want).max()}"
+    # the packed entry point on the separately quantized activation gives the same tensor
+    QX, _ = tab_amd.Quantize(x.cuda(), x_ths.cuda(), act_bits(type), N, H, W, C)
+    y2 = tab_amd.Conv2dPacked(QX, QW, BTN, type, p1, p2, s1, s2, N, H, W, C, KN, KH, KW)
+    assert torch.equal(y, y2)
+
+
+@pytest.mark.parametrize("type", [0, 1, 2, 3])
+def test_config1_shape(type):
+    # BASELINE config 1: N=1, 32x32x64 -> 64, 3x3, pad 1, stride 1
+    _conv_case(type, 1, 32, 32, 64, 64, 3, 3, 1, 1, 1, 1)
+
+
+EDGE_CASES = [
+    # N, H, W, C, KN, KH, KW, p1, p2, s1, s2
+    (2, 7, 7, 64, 8, 3, 3, 1, 1, 2, 2),       # OH = 3 (PyTorch would say 4)
+    (2, 9, 6, 70, 5, 3, 3, 1, 0, 1, 2),       # C % 64 != 0, KN % 4 != 0, asymmetric pad/stride
+    (2, 8, 8, 128, 16, 1, 1, 0, 0, 2, 2),     # 1x1 stride 2
+    (1, 6, 5, 200, 7, 2, 3, 2, 1, 1, 1),      # even kernel, pad > k/2
+    (3, 5, 5, 64, 4, 1, 1, 1, 0, 2, 1),       # 1x1 with padding
+    (1, 3, 3, 64, 1, 3, 3, 0, 0, 1, 1),       # single output element
+    (2, 12, 12, 192, 130, 3, 3, 1, 1, 1, 1),  # KN not a multiple of the 64/128 tile
+    (1, 10, 10, 64, 66, 5, 5, 2, 2, 1, 1),    # 5x5 kernel
+    (5, 4, 4, 1024, 12, 3, 3, 1, 1, 1, 1),    # long K (144 words)
+]
+
+
+@pytest.mark.parametrize("type", [0, 1, 2, 3])
+@pytest.mark.parametrize("case", EDGE_CASES)
+def test_edge_shapes(type, case):
+    _conv_case(type, *case, seed=type + 3, relu=(type == 1))
+
+
+RESNET18_N16 = [
+    # BASELINE configs 2/3: N=16, 3x3 pad 1 stride 1, plus the stride-2 downsample variants
+    (16, 56, 56, 64, 64, 3, 3, 1, 1, 1, 1), (16, 28, 28, 128, 128, 3, 3, 1, 1, 1, 1),
+    (16, 14, 14, 256, 256, 3, 3, 1, 1, 1, 1), (16, 7, 7, 512, 512, 3, 3, 1, 1, 1, 1),
+    (16, 56, 56, 64, 128, 3, 3, 1, 1, 2, 2), (16, 28, 28, 128, 256, 3, 3, 1, 1, 2, 2),
+    (16, 14, 14, 256, 512, 3, 3, 1, 1, 2, 2), (16, 56, 56, 64, 128, 1, 1, 0, 0, 2, 2),
+    (16, 28, 28, 128, 256, 1, 1, 0, 0, 2, 2), (16, 14, 14, 256, 512, 1, 1, 0, 0, 2, 2),
+]
+
+
+@pytest.mark.parametrize("case", RESNET18_N16)
+def test_resnet18_bnn(case):
+    _conv_case(3, *case)
+
+
+@pytest.mark.parametrize("type", [1, 2])
+@pytest.mark.parametrize("case", RESNET18_N16[:4])
+def test_resnet18_tbn_btn_relu_inputs(type, case):
+    _conv_case(type, *case, relu=True)
+
+
+@pytest.mark.parametrize("case", [
+    (1, 28, 28, 512, 512, 3, 3, 1, 1, 1, 1),   # VGG-style 28x28x512 (config 4) at N=1
+    (1, 56, 56, 256, 256, 3, 3, 1, 1, 1, 1),
+    (2, 28, 28, 256, 256, 3, 3, 1, 0, 2, 2),   # sweep shape with asymmetric padding (config 5)
+    (2, 28, 28, 512, 512, 1, 1, 1, 0, 2, 2),
+])
+@pytest.mark.parametrize("type", [0, 1, 2, 3])
+def test_large_channel_layers(type, case):
+    _conv_case(type, *case)
+
+
+def test_arbitrary_weight_bit_patterns():
+    """QW is caller data: the kernels must follow the formulas for any 64-bit pattern, including
+    sign bits outside the nonzero plane (the notebook passes a 1-bit QW to the 2-bit types)."""
+    N, H, W, C, KN, KH, KW = 2, 6, 6, 128, 20, 3, 3
+    rng = np.random.default_rng(0)
+    x, x_ths, _, _ = make_layer(0, N, H, W, C, KN, KH, KW, seed=9)
+    for type in range(4):
+        print(f"[case] random QW bits type={type}", flush=True)
+        qw = rng.integers(-2**63, 2**63 - 1, size=(KN, KH, KW, C // 64, weight_bits(type)), dtype=np.int64, endpoint=True)
+        btn = rng.integers(0, 1000, size=KN).astype(np.int32)
+        ths = x_ths if act_bits(type) == 2 else torch.zeros(N)
+        want = oracle.conv2d(x.numpy(), qw, ths.numpy(), btn, type, 1, 1, 1, 1, N, H, W, C, KN, KH, KW)
+        y = tab_amd.Conv2d(x.cuda(), torch.from_numpy(qw).cuda(), ths.cuda(), torch.from_numpy(btn).cuda(),
+                           type, 1, 1, 1, 1, N, H, W, C, KN, KH, KW)
+        assert np.array_equal(y.cpu().numpy(), want)
+
+
+def test_full_size_sweep_point_properties():
+    """N=256, 28x28x512 -> 512, 3x3 (the largest sweep point, 9.5e11 binary ops) is too slow for
+    the CPU oracle as a whole.  Images are independent, so: the first two images computed alone
+    must equal the same images inside the full batch; the first and the last image are compared
+    with the oracle; and every output obeys |y| <= KH*KW*C and, for BNN, y = NUM (mod 2)."""
+    N, H, W, C, KN = 256, 28, 28, 512, 512
+    print("[case] full-size sweep point N=256 28x28x512->512 3x3 BNN/TNN", flush=True)
+    g = torch.Generator("cuda").manual_seed(0)
+    x = torch.randn((N, H, W, C), generator=g, device="cuda")
+    w = torch.randn((KN, 3, 3, C), generator=g, device="cuda")
+    for type in (3, 0):
+        ab, wb = act_bits(type), weight_bits(type)
+        x_ths = (0.7 * x.abs().reshape(N, -1).mean(dim=1)).contiguous() if ab == 2 else torch.zeros(N, device="cuda")
+        w_ths = (0.7 * w.abs().reshape(KN, -1).mean(dim=1)).contiguous() if wb == 2 else torch.zeros(KN, device="cuda")
+        QW, BTN = tab_amd.Quantize(w, w_ths, wb, KN, 3, 3, C)
+        y = tab_amd.Conv2d(x, QW, x_ths, BTN, type, 1, 1, 1, 1, N, H, W, C, KN, 3, 3)
+        y_small = tab_amd.Conv2d(x[:2].contiguous(), QW, x_ths[:2].contiguous(), BTN, type, 1, 1, 1, 1, 2, H, W, C, KN, 3, 3)
+        torch.cuda.synchronize()
+        assert torch.equal(y[:2], y_small)
+        want = oracle.conv2d(x[:1].cpu().numpy(), QW.cpu().numpy(), x_ths[:1].cpu().numpy(), BTN.cpu().numpy(),
+                             type, 1, 1, 1, 1, 1, H, W, C, KN, 3, 3)
+        assert np.array_equal(y[:1].cpu().numpy(), want)
+        # last image too (a different threshold and the far end of every index range)
+        want_last = oracle.conv2d(x[-1:].cpu().numpy(), QW.cpu().numpy(), x_ths[-1:].cpu().numpy(), BTN.cpu().numpy(),
+                                  type, 1, 1, 1, 1, 1, H, W, C, KN, 3, 3)
+        assert np.array_equal(y[-1:].cpu().numpy(), want_last)
+        assert bool((y.abs() <= 9 * C).all())
+        if type == 3:
+            assert bool(((y.to(torch.int64) - 9 * C) % 2 == 0).all())
+
+
+def test_conv_rejects_wrong_sizes():
+    x = torch.zeros((1, 4, 4, 64), device="cuda")
+    ths = torch.zeros(1, device="cuda")
+    btn = torch.zeros(4, dtype=torch.int32, device="cuda")
+    qw1 = torch.zeros((4, 3, 3, 1, 1), dtype=torch.int64, device="cuda")
+    with pytest.raises(RuntimeError, match="QW has"):
+        tab_amd.Conv2d(x, qw1, ths, btn, 0, 1, 1, 1, 1, 1, 4, 4, 64, 4, 3, 3)  # TNN needs 2-bit QW
+    with pytest.raises(RuntimeError, match="type must be"):
+        tab_amd.Conv2d(x, qw1, ths, btn, 7, 1, 1, 1, 1, 1, 4, 4, 64, 4, 3, 3)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        tab_amd.Conv2d(x.permute(0, 3, 1, 2), qw1, ths, btn, 3, 1, 1, 1, 1, 1, 4, 4, 64, 4, 3, 3)
+    with pytest.raises(RuntimeError, match="dtype"):
+        tab_amd.Conv2d(x.double(), qw1, ths, btn, 3, 1, 1, 1, 1, 1, 4, 4, 64, 4, 3, 3)
+    qw4 = torch.zeros((4, 3, 3, 4, 1), dtype=torch.int64, device="cuda")
+    with pytest.raises(RuntimeError, match="empty output"):
+        tab_amd.Conv2d(x, qw4, ths, btn, 3, 0, 0, 1, 1, 1, 2, 2, 64 * 4, 4, 3, 3)
