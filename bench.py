@@ -1,0 +1,360 @@
+#!/usr/bin/env python3
+"""Benchmark of the TAB hot path on one MI355X.
+
+A step is one pass of Conv2d (quantize + bitwise conv, through the C ABI) over every layer
+of the workload, inputs resident in HBM.  The headline workload is the BNN ResNet-18 layer
+set at N=16; per-layer latencies, the standalone Quantize HBM rate, the large sweep point and
+the CPU oracle's rate are reported in the same JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick]
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+TYPE_NAMES = {0: "TNN", 1: "TBN", 2: "BTN", 3: "BNN"}
+# VALU popcount roofline.  A SIMD issues one wave64 VALU instruction in `cycles`:
+# measured on MI355X with tab_amd/lib/valu_peak (profiles/valu_issue_rates.txt): 2 cycles for
+# v_xor/v_and/v_bitop3 (128 lanes/clk/CU) and 4 cycles for v_bcnt_u32_b32 (64 lanes/clk/CU).
+# Per 32-bit word pair (= 64 binary ops per lane) the kernels issue
+#   BNN xor+bcnt = 6, TBN/BTN bitop3+bcnt = 6, TNN and+bcnt+bitop3+bcnt = 12 cycles.
+# peak = 256 CUs x 4 SIMDs x 2.4 GHz x 64 lanes x 64 binary ops / cycles.
+SIMD_HZ = 256 * 4 * 2.4e9
+ISSUED_CYCLES_PER_PAIR = {0: 12, 1: 6, 2: 6, 3: 6}
+# The planning figure: every op at 64 lanes/clk/CU and the reference's un-fused op mix
+# (TAB_GEMM.cu:48-51,81-84,113-114,142): TNN 5, TBN 4, BTN 3, BNN 2 lane-ops per pair.
+REFERENCE_MIX_OPS = {0: 5, 1: 4, 2: 3, 3: 2}
+HBM_PEAK_GBS = 8000.0
+
+
+def valu_peak_tops(type):
+    """Roofline of the instruction mix the kernel really issues, at the measured issue rates."""
+    return SIMD_HZ * 64 * 64 / ISSUED_CYCLES_PER_PAIR[type] / 1e12
+
+
+def planning_peak_tops(type):
+    """256 CU x 64 lanes x 2.4 GHz lane-ops/s over the reference's op mix."""
+    return 256 * 64 * 2.4e9 * 64 / REFERENCE_MIX_OPS[type] / 1e12
+
+
+# (H, W, C, KN, KH, KW, pad1, pad2, stride1, stride2): ResNet-18 3x3 layers + stride-2 variants
+RESNET18_LAYERS = [
+    (56, 56, 64, 64, 3, 3, 1, 1, 1, 1), (28, 28, 128, 128, 3, 3, 1, 1, 1, 1),
+    (14, 14, 256, 256, 3, 3, 1, 1, 1, 1), (7, 7, 512, 512, 3, 3, 1, 1, 1, 1),
+    (56, 56, 64, 128, 3, 3, 1, 1, 2, 2), (28, 28, 128, 256, 3, 3, 1, 1, 2, 2),
+    (14, 14, 256, 512, 3, 3, 1, 1, 2, 2), (56, 56, 64, 128, 1, 1, 0, 0, 2, 2),
+    (28, 28, 128, 256, 1, 1, 0, 0, 2, 2), (14, 14, 256, 512, 1, 1, 0, 0, 2, 2),
+]
+
+
+def out_extent(size, pad, k, stride):
+    return (size + 2 * pad - k + 1) // stride
+
+
+def layer_ops(N, layer):
+    H, W, C, KN, KH, KW, p1, p2, s1, s2 = layer
+    OH, OW = out_extent(H, p1, KH, s1), out_extent(W, p2, KW, s2)
+    return 2 * N * OH * OW * KN * KH * KW * C
+
+
+def layer_name(N, layer):
+    H, W, C, KN, KH, KW, p1, p2, s1, s2 = layer
+    return f"N{N}_{H}x{W}x{C}->{KN}_k{KH}x{KW}_p{p1}{p2}_s{s1}{s2}"
+
+
+class Layer:
+    """Device-resident inputs of one Conv2d call, built as the benchmark spec says: seeded
+    CPU tensors, X ~ N(0,1) NHWC, W ~ N(0,1), ternary thresholds 0.7*mean|.|, binary 0."""
+
+    def __init__(self, tab, torch, type, N, layer, seed=0, relu=False, on_device=False):
+        H, W, C, KN, KH, KW, p1, p2, s1, s2 = layer
+        self.type, self.N, self.layer = type, N, layer
+        abits = 2 if type < 2 else 1
+        wbits = 2 if type in (0, 2) else 1
+        if on_device:  # shapes too large to generate on the host in reasonable time
+            g = torch.Generator("cuda").manual_seed(seed)
+            x = torch.randn((N, H, W, C), generator=g, device="cuda")
+            w = torch.randn((KN, KH, KW, C), generator=g, device="cuda")
+        else:
+            x = torch.randn((N, H, W, C), generator=torch.Generator("cpu").manual_seed(seed))
+            w = torch.randn((KN, KH, KW, C), generator=torch.Generator("cpu").manual_seed(seed + 1))
+        if relu:
+            x = torch.relu(x)
+        x_ths = 0.7 * x.abs().reshape(N, -1).mean(dim=1) if abits == 2 else torch.zeros(N)
+        w_ths = 0.7 * w.abs().reshape(KN, -1).mean(dim=1) if wbits == 2 else torch.zeros(KN)
+        self.host = None if on_device else (x, x_ths.float(), w, w_ths.float())
+        self.x, self.x_ths = x.cuda().contiguous(), x_ths.float().cuda().contiguous()
+        self.QW, self.BTN = tab.Quantize(w.cuda().contiguous(), w_ths.float().cuda().contiguous(), wbits, KN, KH, KW, C)
+        self.QX, _ = tab.Quantize(self.x, self.x_ths, abits, N, H, W, C)
+        self.abits, self.wbits = abits, wbits
+        self.ops = layer_ops(N, layer)
+        self.args = (type, p1, p2, s1, s2, N, H, W, C, KN, KH, KW)
+        self.tab = tab
+
+    def conv2d(self):
+        return self.tab.Conv2d(self.x, self.QW, self.x_ths, self.BTN, *self.args)
+
+    def conv_kernel_only(self):
+        return self.tab.Conv2dPacked(self.QX, self.QW, self.BTN, *self.args)
+
+    def quantize_only(self):
+        _, p1, p2, s1, s2, N, H, W, C, KN, KH, KW = self.args
+        return self.tab.Quantize(self.x, self.x_ths, self.abits, N, H, W, C)
+
+
+def event_time_ms(torch, fn, reps, warmup=3):
+    """Average duration of fn() over `reps` back-to-back launches, HIP events on the current
+    stream (the stream the library launches on)."""
+    for _ in range(warmup):
+        fn()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(reps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / reps
+
+
+def graph_time_ms(torch, fn, launches, replays=5):
+    """Average duration of fn() when `launches` calls are captured into one HIP graph and the
+    graph is replayed: the launches run back to back on the GPU with no host work between
+    them, so this is the kernel's own duration (what rocprofv3 --kernel-trace reports) plus the
+    dispatch gap.  Timed with HIP events on the stream the graph is launched on."""
+    fn()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(launches):
+            fn()
+    graph.replay()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(replays):
+        graph.replay()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / (replays * launches)
+
+
+def median_call_ms(torch, fn, reps, warmup=3):
+    """Median duration of single fn() calls, each bracketed by its own pair of events."""
+    for _ in range(warmup):
+        fn()
+    times = []
+    for _ in range(reps):
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        fn()
+        stop.record()
+        stop.synchronize()
+        times.append(start.elapsed_time(stop))
+    return statistics.median(times)
+
+
+def cpu_baseline(oracle, layers, check_against=None, budget_s=10.0):
+    """The CPU oracle (this repository's C/OpenMP restatement of the reference's CPU path) over
+    the same layer set and tensors, on the host cores: whole passes until about `budget_s`
+    seconds of CPU work are done, after a small warm-up call."""
+    import numpy as np
+
+    l0 = layers[0]
+    x, x_ths, w, w_ths = (t.numpy() for t in l0.host)
+    _, p1, p2, s1, s2, N, H, W, C, KN, KH, KW = l0.args
+    oracle.conv2d(x[:1], l0.QW.cpu().numpy(), x_ths[:1], l0.BTN.cpu().numpy(), l0.type, p1, p2, s1, s2, 1, H, W, C, KN, KH, KW)
+    total_ops, total_s, exact, passes = 0, 0.0, True, 0
+    host = [[t.numpy() for t in l.host[:2]] + [l.QW.cpu().numpy(), l.BTN.cpu().numpy()] for l in layers]
+    while total_s < budget_s:
+        for i, l in enumerate(layers):
+            x, x_ths, qw, btn = host[i]
+            t0 = time.perf_counter()
+            y = oracle.conv2d(x, qw, x_ths, btn, l.type, *l.args[1:])
+            total_s += time.perf_counter() - t0
+            total_ops += l.ops
+            if check_against is not None and passes == 0:
+                exact = exact and bool(np.array_equal(y, check_against[i]))
+        passes += 1
+    return total_ops / total_s / 1e12, total_s, exact, passes
+
+
+def profile_sequence(torch, tab):
+    """Launch sequence for counter collection: a plain 256 MiB device copy (the yardstick that
+    FETCH_SIZE / WRITE_SIZE are scaled with), Quantize at the roofline shape for both bit
+    widths, the conv kernel of every ResNet-18 N=16 layer, and the conv kernel of the large
+    sweep point for all four types.  Three repetitions each."""
+    src = torch.empty(256 * 1024 * 1024 // 4, dtype=torch.float32, device="cuda").normal_()
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    del src, dst
+    qN, qH, qW, qC = 256, 56, 56, 256
+    xq = torch.randn((qN, qH, qW, qC), generator=torch.Generator("cuda").manual_seed(0), device="cuda")
+    ths = (0.7 * xq.abs().reshape(qN, -1).mean(dim=1)).contiguous()
+    zeros = torch.zeros(qN, device="cuda")
+    for _ in range(3):
+        tab.Quantize(xq, zeros, 1, qN, qH, qW, qC)
+        tab.Quantize(xq, ths, 2, qN, qH, qW, qC)
+    del xq
+    for i, l in enumerate(RESNET18_LAYERS):
+        L = Layer(tab, torch, 3, 16, l, seed=i)
+        for _ in range(3):
+            L.conv_kernel_only()
+    for type in range(4):
+        L = Layer(tab, torch, type, 256, (28, 28, 512, 512, 3, 3, 1, 1, 1, 1), seed=7, on_device=True)
+        for _ in range(3):
+            L.conv_kernel_only()
+        del L
+    torch.cuda.synchronize()
+    print("profile sequence done")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--quick", action="store_true", help="skip the large extra shapes and the CPU baseline")
+    ap.add_argument("--profile", action="store_true",
+                    help="run a short fixed launch sequence for rocprofv3 (kernel trace or one --pmc pass) and exit")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no multi-GPU part (images are independent; "
+              "shard the batch and replicate the weights). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import tab_amd as tab  # raises if the HIP library is not built: there is no fallback
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    if args.profile:
+        profile_sequence(torch, tab)
+        return
+    N = 16
+    layers = [Layer(tab, torch, 3, N, l, seed=i) for i, l in enumerate(RESNET18_LAYERS)]
+    total_ops = sum(l.ops for l in layers)
+
+    def step():
+        for l in layers:
+            l.conv2d()
+
+    # eager: every call goes Python -> C ABI -> launch; host-bound for layers this small
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    eager_elapsed = time.perf_counter() - t0
+
+    # headline: the same step captured once into a HIP graph and replayed (the library only
+    # enqueues kernels on the current stream, so a caller can capture it)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for _ in range(args.warmup):
+        graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    value = total_ops * args.steps / elapsed / 1e12
+
+    # ---- per layer: latency of the whole call, kernel-only rates -------------------------
+    per_layer, conv_ops, conv_ms = [], 0, 0.0
+    for l in layers:
+        call_ms = graph_time_ms(torch, l.conv2d, 20)
+        k_ms = graph_time_ms(torch, l.conv_kernel_only, 20)
+        q_ms = graph_time_ms(torch, l.quantize_only, 20)
+        conv_ops += l.ops
+        conv_ms += k_ms
+        per_layer.append({"layer": layer_name(N, l.layer), "latency_us": round(call_ms * 1e3, 2),
+                          "conv_kernel_us": round(k_ms * 1e3, 2), "quantize_kernel_us": round(q_ms * 1e3, 2),
+                          "conv_kernel_tops": round(l.ops / k_ms / 1e9, 2),
+                          "frac_valu_peak": round(l.ops / k_ms / 1e9 / valu_peak_tops(3), 4)})
+    achieved = conv_ops / conv_ms / 1e9  # TOP/s over the conv launches of one step
+    roofline = {"kernel": "conv_popcount<BNN>", "bound": "valu", "achieved": round(achieved, 2),
+                "peak": round(valu_peak_tops(3), 1), "unit": "TOP/s (effective binary ops)",
+                "frac": round(achieved / valu_peak_tops(3), 4), "traffic": None,
+                "frac_of_planning_peak": round(achieved / planning_peak_tops(3), 4),
+                "planning_peak": round(planning_peak_tops(3), 1),
+                "note": "peak = 1024 SIMDs x 2.4 GHz x 64 lanes x 64 binary ops / 6 issue cycles per 32-bit "
+                        "word pair (v_xor 2 + v_bcnt 4, measured issue rates); planning_peak = 256 CU x 64 "
+                        "lanes x 2.4 GHz / 2 lane-ops per pair; achieved = sum of layer ops / sum of average "
+                        "kernel durations (HIP events around graph replays of 20 launches per layer)"}
+
+    result = {
+        "metric": "tab_conv2d_effective_binary_tops", "value": round(value, 3), "unit": "TOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u32 popcount -> i32 -> f32",
+        "data": "synthetic",
+        "config": {"workload": "BNN (type 3) ResNet-18 layer set, N=16: 4x 3x3 s1 + 3x 3x3 s2 + 3x 1x1 s2; "
+                               "one step = Conv2d (quantize + conv) on all 10 layers, replayed as one HIP graph",
+                   "binary_ops_per_step": total_ops},
+        "eager": {"tops": round(total_ops * args.steps / eager_elapsed / 1e12, 3),
+                  "ms_per_step": round(eager_elapsed / args.steps * 1e3, 4),
+                  "note": "same step launched call by call from Python (host-bound)"},
+        "roofline": roofline, "per_layer": per_layer,
+    }
+
+    # ---- standalone Quantize at the HBM-roofline shape -------------------------------------
+    if not args.quick:
+        qN, qH, qW, qC = 256, 56, 56, 256
+        xq = torch.randn((qN, qH, qW, qC), generator=torch.Generator("cuda").manual_seed(0), device="cuda")
+        quant = {}
+        for bitwidth in (1, 2):
+            ths = (0.7 * xq.abs().reshape(qN, -1).mean(dim=1)).contiguous() if bitwidth == 2 else torch.zeros(qN, device="cuda")
+            ms = event_time_ms(torch, lambda: tab.Quantize(xq, ths, bitwidth, qN, qH, qW, qC), 20)
+            nbytes = 4 * qN * qH * qW * qC + 8 * qN * qH * qW * (qC // 64) * bitwidth + 8 * qN
+            quant[f"bitwidth{bitwidth}"] = {"us": round(ms * 1e3, 1), "GBps": round(nbytes / ms / 1e6, 1),
+                                            "frac_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
+                                            "bytes": nbytes}
+        del xq
+        result["quantize"] = {"shape": "256x56x56x256 fp32", "bound": "hbm", "peak_GBps": HBM_PEAK_GBS, **quant}
+
+        # ---- the largest sweep point, all four types (conv kernel only) --------------------
+        big = (28, 28, 512, 512, 3, 3, 1, 1, 1, 1)
+        sweep = {}
+        for type in range(4):
+            L = Layer(tab, torch, type, 256, big, seed=7, relu=(type == 1), on_device=True)
+            k_ms = event_time_ms(torch, L.conv_kernel_only, 5, warmup=2)
+            call_ms = median_call_ms(torch, L.conv2d, 5, warmup=1)
+            sweep[TYPE_NAMES[type]] = {"conv_kernel_ms": round(k_ms, 3), "call_ms": round(call_ms, 3),
+                                       "conv_kernel_tops": round(L.ops / k_ms / 1e9, 1),
+                                       "valu_peak_tops": round(valu_peak_tops(type), 1),
+                                       "frac_valu_peak": round(L.ops / k_ms / 1e9 / valu_peak_tops(type), 4),
+                                       "planning_peak_tops": round(planning_peak_tops(type), 1),
+                                       "frac_of_planning_peak": round(L.ops / k_ms / 1e9 / planning_peak_tops(type), 4)}
+            del L
+        result["sweep_N256_28x28x512_3x3"] = sweep
+
+        # ---- CPU baseline: the oracle on the same layer set, same tensors --------------------
+        import oracle
+
+        gpu_out = [l.conv2d().cpu().numpy() for l in layers]
+        tops, secs, exact, passes = cpu_baseline(oracle, layers, gpu_out)
+        result["cpu_baseline"] = {"value": round(tops, 4), "unit": "TOP/s", "cores": oracle.num_threads(),
+                                  "kind": "port",
+                                  "sample": f"the full workload (10 layers, N=16, {total_ops:.3e} binary ops per pass), "
+                                            f"{passes} passes in {secs:.2f} s: quantize + pad + im2row + popcount GEMM, "
+                                            "OpenMP over rows",
+                                  "gpu_bit_exact_vs_cpu": exact}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -13,6 +13,20 @@ HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
+PEAK_SRC = os.path.join(CSRC, "valu_peak.hip")
+PEAK_BIN = os.path.join(LIB_DIR, "valu_peak")
+
+
+def build_valu_peak():
+    """Standalone microbenchmark of the VALU issue rates the conv roofline is priced with."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    cmd = [HIPCC] + HIP_FLAGS + ["-o", PEAK_BIN, PEAK_SRC]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + proc.stdout)
+    return PEAK_BIN
+
+
 def build_library(verbose=False):
     """Compile every HIP source and link libtab_amd.so. Always recompiles."""
     os.makedirs(LIB_DIR, exist_ok=True)
@@ -28,3 +42,4 @@ def build_library(verbose=False):
 
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_valu_peak())

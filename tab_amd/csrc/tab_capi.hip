@@ -75,6 +75,9 @@ const char *tab_last_error(void) { return g_last_error; }
 
 const char *tab_version(void) { return "tab_amd 0.1 gfx950"; }
 
+/* Tuning hook for benchmarking scripts; deliberately absent from include/tab_amd.h. */
+void tab_internal_force_conv_tile(int tm, int ng) { tab::force_conv_tile(tm, ng); }
+
 int tab_packed_channels(int C) { return (C + tab::kWordBits - 1) / tab::kWordBits; }
 
 int tab_out_extent(int in, int pad, int k, int stride)

@@ -52,4 +52,6 @@ hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream);
 hipError_t launch_quantize(const float *x, const float *ths, int bitwidth, long pixels_per_item,
                            long items, int C, uint64_t *qx, int32_t *btn, hipStream_t stream);
 
+void force_conv_tile(int tm, int ng);  // tuning hook: 0,0 restores the automatic choice
+
 }  // namespace tab

@@ -64,6 +64,19 @@ __device__ __forceinline__ void store_item(uint32_t *lds, const Item<PL> &it, in
             lds[((pl * kMaxQ) + 2 * word + half) * ROWS + row] = it.d[pl * 2 + half];
 }
 
+// acc += popcount(x) as the single instruction v_bcnt_u32_b32 (count + addend).  Kept opaque
+// so the compiler cannot re-associate two counts into bcnt(x,0) + bcnt(y,0) + add3.
+__device__ __forceinline__ void popcount_acc(int &acc, uint32_t x)
+{
+    asm("v_bcnt_u32_b32 %0, %1, %0" : "+v"(acc) : "v"(x));
+}
+
+// (x ^ y) & m in one gfx950 v_bitop3_b32 (truth table 0x28 with the operands as 0xF0, 0xCC, 0xAA).
+__device__ __forceinline__ uint32_t xor_and(uint32_t x, uint32_t y, uint32_t m)
+{
+    return __builtin_amdgcn_bitop3_b32(x, y, m, 0x28);
+}
+
 template <int TYPE, int TM, int NG>
 __global__ __launch_bounds__(kThreads) void conv_popcount(const ConvArgs p)
 {
@@ -77,7 +90,8 @@ __global__ __launch_bounds__(kThreads) void conv_popcount(const ConvArgs p)
     static_assert(kThreads % BM == 0 && kThreads % BN == 0, "tile rows must divide the workgroup");
     static_assert(TM % 4 == 0 || TM == 2, "TM is read with 64- or 128-bit LDS loads");
 
-    __shared__ __attribute__((aligned(16))) uint32_t lds[2][A_DWORDS + B_DWORDS];
+    // + one spare k-slice of the wider operand: the pipelined loop reads one slice ahead
+    __shared__ __attribute__((aligned(16))) uint32_t lds[2 * (A_DWORDS + B_DWORDS) + (BM > BN ? BM : BN)];
 
     const int tid = threadIdx.x;
     const int tx = tid & 15, ty = tid >> 4;
@@ -135,7 +149,7 @@ __global__ __launch_bounds__(kThreads) void conv_popcount(const ConvArgs p)
         }
     };
     auto stage = [&](int buf) {
-        uint32_t *la = lds[buf], *lb = lds[buf] + A_DWORDS;
+        uint32_t *la = lds + buf * (A_DWORDS + B_DWORDS), *lb = la + A_DWORDS;
 #pragma unroll
         for (int i = 0; i < A_ITEMS; i++) {
             const int w = a_w0 + i * A_STEP;
@@ -166,6 +180,62 @@ __global__ __launch_bounds__(kThreads) void conv_popcount(const ConvArgs p)
         for (int i = 0; i < TM; i++) row_nz[i] = 0;
     }
 
+    // One k-slice (32 bits of K) of this thread's operands.
+    struct Frag {
+        uint32_t a[APL][TM], b[BPL][TN];
+    };
+    auto read_frag = [&](Frag &f, const uint32_t *la, const uint32_t *lb, int q) {
+#pragma unroll
+        for (int pl = 0; pl < APL; pl++) {
+            const uint32_t *src = la + (pl * kMaxQ + q) * BM + ty * TM;
+            if (TM == 2) {
+                const u32x2 v = *reinterpret_cast<const u32x2 *>(src);
+                f.a[pl][0] = v[0]; f.a[pl][1] = v[1];
+            } else {
+#pragma unroll
+                for (int i4 = 0; i4 < TM / 4; i4++) {
+                    const u32x4 v = *reinterpret_cast<const u32x4 *>(src + 4 * i4);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) f.a[pl][4 * i4 + e] = v[e];
+                }
+            }
+        }
+#pragma unroll
+        for (int pl = 0; pl < BPL; pl++)
+#pragma unroll
+            for (int g = 0; g < NG; g++) {
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(lb + (pl * kMaxQ + q) * BN + g * 64 + tx * 4);
+#pragma unroll
+                for (int e = 0; e < 4; e++) f.b[pl][4 * g + e] = v[e];
+            }
+    };
+    auto mac = [&](const Frag &f) {
+        if (TYPE == 1) {
+#pragma unroll
+            for (int i = 0; i < TM; i++) popcount_acc(row_nz[i], f.a[APL - 1][i]);
+        }
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                if (TYPE == 0) {
+                    // TAB_GEMM.cu:48-51
+                    const uint32_t both = f.a[1][i] & f.b[1][j];
+                    popcount_acc(nzc[i][j], both);
+                    popcount_acc(acc[i][j], xor_and(f.a[0][i], f.b[0][j], both));
+                } else if (TYPE == 1) {
+                    // TAB_GEMM.cu:81-84; popcount(a1) is summed once per row above
+                    popcount_acc(acc[i][j], xor_and(f.a[0][i], f.b[0][j], f.a[1][i]));
+                } else if (TYPE == 2) {
+                    // TAB_GEMM.cu:113-114
+                    popcount_acc(acc[i][j], xor_and(f.a[0][i], f.b[0][j], f.b[1][j]));
+                } else {
+                    // TAB_GEMM.cu:142
+                    popcount_acc(acc[i][j], f.a[0][i] ^ f.b[0][j]);
+                }
+            }
+    };
+
     fetch(0);
     stage(0);
     __syncthreads();
@@ -174,59 +244,27 @@ __global__ __launch_bounds__(kThreads) void conv_popcount(const ConvArgs p)
         const bool more = chunk + 1 < p.nchunks;
         if (more) fetch(chunk + 1);
 
-        const uint32_t *la = lds[chunk & 1], *lb = lds[chunk & 1] + A_DWORDS;
+        const uint32_t *la = lds + (chunk & 1) * (A_DWORDS + B_DWORDS), *lb = la + A_DWORDS;
         const int words_here = (p.G - chunk * p.kcw < p.kcw) ? p.G - chunk * p.kcw : p.kcw;
         const int nq = 2 * words_here;
-        for (int q = 0; q < nq; q++) {
-            uint32_t a[APL][TM], b[BPL][TN];
-#pragma unroll
-            for (int pl = 0; pl < APL; pl++) {
-                const uint32_t *src = la + (pl * kMaxQ + q) * BM + ty * TM;
-                if (TM == 2) {
-                    const u32x2 v = *reinterpret_cast<const u32x2 *>(src);
-                    a[pl][0] = v[0]; a[pl][1] = v[1];
-                } else {
-#pragma unroll
-                    for (int i4 = 0; i4 < TM / 4; i4++) {
-                        const u32x4 v = *reinterpret_cast<const u32x4 *>(src + 4 * i4);
-#pragma unroll
-                        for (int e = 0; e < 4; e++) a[pl][4 * i4 + e] = v[e];
-                    }
-                }
-            }
-#pragma unroll
-            for (int pl = 0; pl < BPL; pl++)
-#pragma unroll
-                for (int g = 0; g < NG; g++) {
-                    const u32x4 v = *reinterpret_cast<const u32x4 *>(lb + (pl * kMaxQ + q) * BN + g * 64 + tx * 4);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) b[pl][4 * g + e] = v[e];
-                }
-
-            if (TYPE == 1) {
-#pragma unroll
-                for (int i = 0; i < TM; i++) row_nz[i] += __builtin_popcount(a[APL - 1][i]);
-            }
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++) {
-                    if (TYPE == 0) {
-                        // TAB_GEMM.cu:48-51
-                        const uint32_t both = a[1][i] & b[1][j];
-                        nzc[i][j] += __builtin_popcount(both);
-                        acc[i][j] += __builtin_popcount((a[0][i] ^ b[0][j]) & both);
-                    } else if (TYPE == 1) {
-                        // TAB_GEMM.cu:81-84; popcount(a1) is summed once per row above
-                        acc[i][j] += __builtin_popcount((a[0][i] ^ b[0][j]) & a[1][i]);
-                    } else if (TYPE == 2) {
-                        // TAB_GEMM.cu:113-114
-                        acc[i][j] += __builtin_popcount((a[0][i] ^ b[0][j]) & b[1][j]);
-                    } else {
-                        // TAB_GEMM.cu:142
-                        acc[i][j] += __builtin_popcount(a[0][i] ^ b[0][j]);
-                    }
-                }
+        // Register double buffering: the LDS reads of k-slice q+1 are issued before the VALU
+        // work of slice q, so a single wave per SIMD still keeps the VALU busy.  nq is even.
+        // The read of slice nq after the last pair stays inside the LDS allocation (one spare
+        // slice is reserved) and its value is never used.
+        Frag f0, f1;
+        // drain outstanding scalar loads first: they share the LDS counter and return out of
+        // order, which would force full waits inside the loop
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        read_frag(f0, la, lb, 0);
+        for (int q = 0; q < nq; q += 2) {
+            read_frag(f1, la, lb, q + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            mac(f0);
+            __builtin_amdgcn_sched_barrier(0);
+            read_frag(f0, la, lb, q + 2);
+            __builtin_amdgcn_sched_barrier(0);
+            mac(f1);
+            __builtin_amdgcn_sched_barrier(0);
         }
 
         if (more) stage((chunk + 1) & 1);
@@ -282,11 +320,21 @@ hipError_t launch_tile(ConvArgs a, hipStream_t stream)
     return hipGetLastError();
 }
 
+// Tuning hook (not part of the public ABI): forces one tile shape for every launch.
+int g_force_tm = 0, g_force_ng = 0;
+
 // Tile choice: the largest tile that still gives every CU a few workgroups; small layers
 // fall back to smaller tiles so that the 256 CUs are not left idle.
 template <int TYPE>
 hipError_t launch_type(const ConvArgs &a, hipStream_t stream)
 {
+    if (g_force_tm) {
+        const int ng = (TYPE == 0) ? 1 : g_force_ng;
+        if (g_force_tm == 8 && ng == 2) return launch_tile<TYPE, 8, (TYPE == 0 ? 1 : 2)>(a, stream);
+        if (g_force_tm == 8) return launch_tile<TYPE, 8, 1>(a, stream);
+        if (g_force_tm == 4) return launch_tile<TYPE, 4, 1>(a, stream);
+        return launch_tile<TYPE, 2, 1>(a, stream);
+    }
     const long want = 2 * 256;  // at least two workgroups per CU
     auto tiles = [&](int bm, int bn) { return (long)((a.M + bm - 1) / bm) * ((a.KN + bn - 1) / bn); };
     if (TYPE != 0 && a.KN > 64 && tiles(128, 128) >= want) return launch_tile<TYPE, 8, (TYPE == 0 ? 1 : 2)>(a, stream);
@@ -296,6 +344,12 @@ hipError_t launch_type(const ConvArgs &a, hipStream_t stream)
 }
 
 }  // namespace
+
+void force_conv_tile(int tm, int ng)
+{
+    g_force_tm = tm;
+    g_force_ng = ng;
+}
 
 hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream)
 {

@@ -61,11 +61,10 @@ __device__ __forceinline__ void compare4(const floatx4 v, const float t, uint32_
 // a wave reads 4 consecutive rows per load (1 KB contiguous) and keeps kLoadsPerLane loads
 // in flight.  Each lane turns its 4 compares into a nibble placed at bit 4*(lane%8); an OR
 // over 8 lanes yields the low (lanes 0-7) or high (lanes 8-15) 32 bits of the word.
-template <int BITS, bool WITH_BTN>
+template <int BITS>
 __global__ __launch_bounds__(kThreads) void quantize_rows64(const floatx4 *__restrict__ x,
                                                             const float *__restrict__ ths,
-                                                            uint32_t *__restrict__ q,
-                                                            int32_t *__restrict__ btn, long rows,
+                                                            uint32_t *__restrict__ q, long rows,
                                                             long rows_per_item)
 {
     const int lane = threadIdx.x & 63;
@@ -74,7 +73,8 @@ __global__ __launch_bounds__(kThreads) void quantize_rows64(const floatx4 *__res
     const int l = lane & 15;    // float4 within the row
     const long row0 = ((long)blockIdx.x * kWavesPerBlock + wave) * kRowsPerWave;
     if (row0 >= rows) return;
-    const long row_last = (row0 + kRowsPerWave - 1 < rows ? row0 + kRowsPerWave - 1 : rows - 1);
+    long row_last = row0 + kRowsPerWave - 1;
+    if (row_last > rows - 1) row_last = rows - 1;
 
     floatx4 v[kLoadsPerLane];
 #pragma unroll
@@ -86,30 +86,18 @@ __global__ __launch_bounds__(kThreads) void quantize_rows64(const floatx4 *__res
     const long item_first = row0 / rows_per_item;
     const bool one_item = (row_last / rows_per_item) == item_first;  // wave-uniform
     const float t_first = ths[item_first];
-    int count = 0;
 
 #pragma unroll
     for (int u = 0; u < kLoadsPerLane; u++) {
         const long r = row0 + u * 4 + sub;
         float t = t_first;
-        long item = item_first;
-        if (!one_item) {
-            item = (r < rows ? r : rows - 1) / rows_per_item;
-            t = ths[item];
-        }
+        if (!one_item) t = ths[(r < rows ? r : rows - 1) / rows_per_item];
         uint32_t sign, nz;
         compare4<BITS>(v[u], t, sign, nz);
         const int shift = 4 * (l & 7);
         const uint32_t sign_word = or_reduce8(sign << shift);
         if (BITS == 2) {
             const uint32_t nz_word = or_reduce8(nz << shift);
-            if (WITH_BTN) {
-                if (one_item) {
-                    count += __builtin_popcount(nz);
-                } else if (r < rows && nz) {
-                    atomicAdd(&btn[item], __builtin_popcount(nz));
-                }
-            }
             // dword (r*2 + plane)*2 + half; lanes 0/1 of each half-row store plane 0/1
             if (r < rows && (l & 7) < 2) {
                 const int plane = l & 1, half = l >> 3;
@@ -119,21 +107,16 @@ __global__ __launch_bounds__(kThreads) void quantize_rows64(const floatx4 *__res
             if (r < rows && (l & 7) == 0) q[r * 2 + (l >> 3)] = sign_word;
         }
     }
-    if (BITS == 2 && WITH_BTN && one_item) {
-        count = wave_sum(count);
-        if (lane == 0 && count) atomicAdd(&btn[item_first], count);
-    }
 }
 
 // General path (any C, any alignment): one wave per (pixel, word); lane i tests channel
 // word*64 + i and the two wave-wide ballots are the packed words, LSB first
 // (onebit[i] = 1 << i, TAB_GEMM.cu:252-258).  Unused high bits of a tail word stay 0
 // (TAB_GEMM.cu:203-206).
-template <int BITS, bool WITH_BTN>
+template <int BITS>
 __global__ __launch_bounds__(kThreads) void quantize_ballot(const float *__restrict__ x,
                                                             const float *__restrict__ ths,
-                                                            uint64_t *__restrict__ q,
-                                                            int32_t *__restrict__ btn, long pixels,
+                                                            uint64_t *__restrict__ q, long pixels,
                                                             long pixels_per_item, int C, int PC)
 {
     const int lane = threadIdx.x & 63;
@@ -155,7 +138,6 @@ __global__ __launch_bounds__(kThreads) void quantize_ballot(const float *__restr
             if (lane == 0) {
                 q[unit * 2 + 0] = sign;
                 q[unit * 2 + 1] = nz;
-                if (WITH_BTN && nz) atomicAdd(&btn[item], __popcll(nz));
             }
         } else {
             const uint64_t neg = __ballot(live && (v < t));
@@ -170,6 +152,39 @@ __global__ void fill_zero_i32(int32_t *p, long n)
     if (i < n) p[i] = 0;
 }
 
+// btn[n] = sum over item n of popcount(nonzero-plane word) (BTN_Weight, TAB_GEMM.cu:150-160,
+// for every n).  q is the ternary output [items][words_per_item][2]; one workgroup per
+// (item, split) reads its words as 16-byte (sign, nonzero) pairs.  With one split the result
+// is stored directly; with several (very long items) the partial sums are added atomically
+// into btn, which the caller zeroed beforehand.
+__global__ __launch_bounds__(kThreads) void btn_popcount(const ulonglong2 *__restrict__ q,
+                                                         int32_t *__restrict__ btn,
+                                                         long words_per_item, int splits)
+{
+    __shared__ int partial[kWavesPerBlock];
+    const long item = blockIdx.x / splits;
+    const int split = blockIdx.x % splits;
+    const long per_split = (words_per_item + splits - 1) / splits;
+    const long w0 = split * per_split;
+    long w1 = w0 + per_split;
+    if (w1 > words_per_item) w1 = words_per_item;
+    const ulonglong2 *src = q + item * words_per_item;
+    int count = 0;
+    for (long w = w0 + threadIdx.x; w < w1; w += kThreads) count += __popcll(src[w].y);
+    count = wave_sum(count);
+    if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = count;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int total = 0;
+#pragma unroll
+        for (int w = 0; w < kWavesPerBlock; w++) total += partial[w];
+        if (splits == 1)
+            btn[item] = total;
+        else if (total)
+            atomicAdd(&btn[item], total);
+    }
+}
+
 }  // namespace
 
 // x: fp32 [items][pixels_per_item][C]; qx: [items*pixels_per_item][PC][bitwidth];
@@ -179,40 +194,41 @@ hipError_t launch_quantize(const float *x, const float *ths, int bitwidth, long 
 {
     const int PC = (C + kWordBits - 1) / kWordBits;
     const long pixels = items * pixels_per_item;
-    if (btn) {
-        // zero with a kernel, not a memset node, so callers may capture the call in a graph
+    const long words_per_item = pixels_per_item * PC;
+    // very long items are split over several workgroups for the btn pass
+    int splits = 1;
+    if (btn && bitwidth == 2 && items < 512) {
+        while (splits < 64 && items * splits < 512 && words_per_item / (splits * 2) >= 16 * kThreads) splits *= 2;
+    }
+    if (btn && (bitwidth != 2 || splits > 1)) {
+        // zeros for 1-bit (TAB_GEMM.cu:283); a kernel rather than a memset node so that the
+        // call can be captured in a graph
         fill_zero_i32<<<dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream>>>(btn, items);
     }
-    const bool want_btn = btn != nullptr && bitwidth == 2;
     const bool fast = (C % kWordBits == 0) && ((uintptr_t)x % 16 == 0);
     if (fast) {
         const long rows = pixels * PC;
-        const long rows_per_item = pixels_per_item * PC;
         const long blocks = (rows + kRowsPerWave * kWavesPerBlock - 1) / (kRowsPerWave * kWavesPerBlock);
         const dim3 grid((unsigned)blocks), block(kThreads);
         const floatx4 *x4 = reinterpret_cast<const floatx4 *>(x);
         uint32_t *q32 = reinterpret_cast<uint32_t *>(qx);
-        if (bitwidth == 2) {
-            if (want_btn)
-                quantize_rows64<2, true><<<grid, block, 0, stream>>>(x4, ths, q32, btn, rows, rows_per_item);
-            else
-                quantize_rows64<2, false><<<grid, block, 0, stream>>>(x4, ths, q32, btn, rows, rows_per_item);
-        } else {
-            quantize_rows64<1, false><<<grid, block, 0, stream>>>(x4, ths, q32, btn, rows, rows_per_item);
-        }
+        if (bitwidth == 2)
+            quantize_rows64<2><<<grid, block, 0, stream>>>(x4, ths, q32, rows, words_per_item);
+        else
+            quantize_rows64<1><<<grid, block, 0, stream>>>(x4, ths, q32, rows, words_per_item);
     } else {
         const long units = pixels * PC;
         long blocks = (units + kWavesPerBlock - 1) / kWavesPerBlock;
         if (blocks > 256 * 32) blocks = 256 * 32;  // grid-stride beyond 32 blocks per CU
         const dim3 grid((unsigned)blocks), block(kThreads);
-        if (bitwidth == 2) {
-            if (want_btn)
-                quantize_ballot<2, true><<<grid, block, 0, stream>>>(x, ths, qx, btn, pixels, pixels_per_item, C, PC);
-            else
-                quantize_ballot<2, false><<<grid, block, 0, stream>>>(x, ths, qx, btn, pixels, pixels_per_item, C, PC);
-        } else {
-            quantize_ballot<1, false><<<grid, block, 0, stream>>>(x, ths, qx, btn, pixels, pixels_per_item, C, PC);
-        }
+        if (bitwidth == 2)
+            quantize_ballot<2><<<grid, block, 0, stream>>>(x, ths, qx, pixels, pixels_per_item, C, PC);
+        else
+            quantize_ballot<1><<<grid, block, 0, stream>>>(x, ths, qx, pixels, pixels_per_item, C, PC);
+    }
+    if (btn && bitwidth == 2) {
+        btn_popcount<<<dim3((unsigned)(items * splits)), dim3(kThreads), 0, stream>>>(
+            reinterpret_cast<const ulonglong2 *>(qx), btn, words_per_item, splits);
     }
     return hipGetLastError();
 }
