@@ -27,6 +27,37 @@ def build_valu_peak():
     return PEAK_BIN
 
 
+def extension_path():
+    import sysconfig
+
+    return os.path.join(HERE, "_C" + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def build_torch_extension(verbose=False):
+    """Compile csrc/torch_binding.cpp (host code only: g++, no hipify, no HIP sources) into the
+    CPython extension tab_amd/_C, linked against libtab_amd.so and the torch libraries."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension
+
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    includes = cpp_extension.include_paths() + [sysconfig.get_paths()["include"], "/opt/rocm/include"]
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           "-DTORCH_EXTENSION_NAME=_C", "-DTORCH_API_INCLUDE_EXTENSION_H",
+           "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI)]
+    cmd += ["-I" + i for i in includes]
+    cmd += [os.path.join(CSRC, "torch_binding.cpp"), "-o", extension_path(), "-L" + torch_lib, "-L" + LIB_DIR,
+            "-ltab_amd", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch", "-ltorch_python",
+            "-Wl,-rpath,$ORIGIN/lib", "-Wl,-rpath," + torch_lib]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("g++ failed:\n" + proc.stdout)
+    if verbose and proc.stdout.strip():
+        print(proc.stdout)
+    return extension_path()
+
+
 def build_library(verbose=False):
     """Compile every HIP source and link libtab_amd.so. Always recompiles."""
     os.makedirs(LIB_DIR, exist_ok=True)
@@ -43,3 +74,4 @@ def build_library(verbose=False):
 if __name__ == "__main__":
     print(build_library(verbose=True))
     print(build_valu_peak())
+    print(build_torch_extension(verbose=True))

@@ -87,3 +87,14 @@ def test_python_mirror_names_and_input_checks():
 def test_missing_library_fails_loudly(tmp_path):
     with pytest.raises(ImportError, match="no fallback"):
         _capi.load(str(tmp_path / "libtab_amd.so"))
+
+
+def test_extension_module_names_and_cpu_rejection():
+    """The pybind module exports the reference's names (TAB_GPU.cpp:62-65) and applies
+    CHECK_INPUT (TAB_GPU.cpp:7-9) before touching the device."""
+    import TAB_CUDA as TAB
+
+    public = [n for n in dir(TAB) if not n.startswith("_")]
+    assert "Conv2d" in public and "Quantize" in public
+    with pytest.raises(RuntimeError, match="X must be a CUDA tensor"):
+        TAB.Quantize(torch.zeros(1, 4, 4, 64), torch.zeros(1), 2, 1, 4, 4, 64)
