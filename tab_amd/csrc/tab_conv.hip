@@ -19,8 +19,6 @@ namespace tab {
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kMaxChunkWords = 8;             // packed 64-bit words of K per chunk, at most
-constexpr int kMaxQ = 2 * kMaxChunkWords;     // 32-bit k-slices per chunk
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -53,35 +51,81 @@ __device__ __forceinline__ Item<PL> load_item(const uint64_t *p, bool valid)
     return it;
 }
 
-// LDS placement: dword index ((plane*kMaxQ + q) * ROWS + row)
-template <int PL, int ROWS>
+// LDS placement: dword index ((plane*Q + q) * ROWS + row), Q = 32-bit k-slices per chunk
+template <int PL, int ROWS, int Q>
 __device__ __forceinline__ void store_item(uint32_t *lds, const Item<PL> &it, int word, int row)
 {
 #pragma unroll
     for (int pl = 0; pl < PL; pl++)
 #pragma unroll
         for (int half = 0; half < 2; half++)
-            lds[((pl * kMaxQ) + 2 * word + half) * ROWS + row] = it.d[pl * 2 + half];
+            lds[((pl * Q) + 2 * word + half) * ROWS + row] = it.d[pl * 2 + half];
 }
 
-// acc += popcount(x) as the single instruction v_bcnt_u32_b32 (count + addend).  Kept opaque
-// so the compiler cannot re-associate two counts into bcnt(x,0) + bcnt(y,0) + add3.
+// Inner-loop primitives.  Measured on MI355X (tab_amd/lib/valu_peak and register-level probes):
+// a SIMD issues v_xor/v_and/v_bitop3 in 2 cycles and v_bcnt_u32_b32 in 4, but only when one
+// scalar `s_nop 0` sits between the logic op and its v_bcnt (xor+bcnt back to back: 8.6 cycles
+// per wave; xor, s_nop, bcnt: 6.4; a nop after the bcnt as well: 8.4 again), and only with an
+// even number of waves per SIMD.  The compiler puts a nop of its own between any two asm
+// statements, so each statement below covers four word pairs of one row: (logic, nop, bcnt) x 4.
+// v_bcnt carries the accumulator as its addend.
+#define TAB_XB(n) "v_xor_b32 %[t], %[a], %[b" #n "]\n\ts_nop 0\n\tv_bcnt_u32_b32 %[c" #n "], %[t], %[c" #n "]\n\t"
+#define TAB_TB(n, m) \
+    "v_bitop3_b32 %[t], %[a], %[b" #n "], %[" m "] bitop3:0x28\n\ts_nop 0\n\tv_bcnt_u32_b32 %[c" #n "], %[t], %[c" #n "]\n\t"
+#define TAB_TNN(n)                                                                                            \
+    "v_and_b32 %[u], %[a1], %[m" #n "]\n\ts_nop 0\n\tv_bcnt_u32_b32 %[z" #n "], %[u], %[z" #n "]\n\t"         \
+    "v_bitop3_b32 %[t], %[a], %[b" #n "], %[u] bitop3:0x28\n\ts_nop 0\n\tv_bcnt_u32_b32 %[c" #n "], %[t], %[c" #n "]\n\t"
+
+// c[j] += popcount(a ^ b[j]), j = 0..3                                        (BNN, TAB_GEMM.cu:142)
+__device__ __forceinline__ void bnn_quad(int *c, uint32_t a, const uint32_t *b)
+{
+    uint32_t t;
+    asm(TAB_XB(0) TAB_XB(1) TAB_XB(2) TAB_XB(3)
+        : [c0] "+v"(c[0]), [c1] "+v"(c[1]), [c2] "+v"(c[2]), [c3] "+v"(c[3]), [t] "=&v"(t)
+        : [a] "v"(a), [b0] "v"(b[0]), [b1] "v"(b[1]), [b2] "v"(b[2]), [b3] "v"(b[3]));
+}
+// c[j] += popcount((a ^ b[j]) & m), j = 0..3: one v_bitop3_b32 (truth table 0x28 for operands
+// 0xF0, 0xCC, 0xAA) per pair                                             (TBN, TAB_GEMM.cu:81-84)
+__device__ __forceinline__ void tbn_quad(int *c, uint32_t a, uint32_t m, const uint32_t *b)
+{
+    uint32_t t;
+    asm(TAB_TB(0, "m") TAB_TB(1, "m") TAB_TB(2, "m") TAB_TB(3, "m")
+        : [c0] "+v"(c[0]), [c1] "+v"(c[1]), [c2] "+v"(c[2]), [c3] "+v"(c[3]), [t] "=&v"(t)
+        : [a] "v"(a), [m] "v"(m), [b0] "v"(b[0]), [b1] "v"(b[1]), [b2] "v"(b[2]), [b3] "v"(b[3]));
+}
+// c[j] += popcount((a ^ b[j]) & m[j]), j = 0..3                          (BTN, TAB_GEMM.cu:113-114)
+__device__ __forceinline__ void btn_quad(int *c, uint32_t a, const uint32_t *b, const uint32_t *m)
+{
+    uint32_t t;
+    asm(TAB_TB(0, "m0") TAB_TB(1, "m1") TAB_TB(2, "m2") TAB_TB(3, "m3")
+        : [c0] "+v"(c[0]), [c1] "+v"(c[1]), [c2] "+v"(c[2]), [c3] "+v"(c[3]), [t] "=&v"(t)
+        : [a] "v"(a), [b0] "v"(b[0]), [b1] "v"(b[1]), [b2] "v"(b[2]), [b3] "v"(b[3]), [m0] "v"(m[0]),
+          [m1] "v"(m[1]), [m2] "v"(m[2]), [m3] "v"(m[3]));
+}
+// both = a1 & m[j]; z[j] += popcount(both); c[j] += popcount((a ^ b[j]) & both)   (TNN, TAB_GEMM.cu:48-51)
+__device__ __forceinline__ void tnn_quad(int *z, int *c, uint32_t a, uint32_t a1, const uint32_t *b, const uint32_t *m)
+{
+    uint32_t t, u;
+    asm(TAB_TNN(0) TAB_TNN(1) TAB_TNN(2) TAB_TNN(3)
+        : [z0] "+v"(z[0]), [z1] "+v"(z[1]), [z2] "+v"(z[2]), [z3] "+v"(z[3]), [c0] "+v"(c[0]), [c1] "+v"(c[1]),
+          [c2] "+v"(c[2]), [c3] "+v"(c[3]), [t] "=&v"(t), [u] "=&v"(u)
+        : [a] "v"(a), [a1] "v"(a1), [b0] "v"(b[0]), [b1] "v"(b[1]), [b2] "v"(b[2]), [b3] "v"(b[3]), [m0] "v"(m[0]),
+          [m1] "v"(m[1]), [m2] "v"(m[2]), [m3] "v"(m[3]));
+}
+// acc += popcount(x)
 __device__ __forceinline__ void popcount_acc(int &acc, uint32_t x)
 {
     asm("v_bcnt_u32_b32 %0, %1, %0" : "+v"(acc) : "v"(x));
 }
 
-// (x ^ y) & m in one gfx950 v_bitop3_b32 (truth table 0x28 with the operands as 0xF0, 0xCC, 0xAA).
-__device__ __forceinline__ uint32_t xor_and(uint32_t x, uint32_t y, uint32_t m)
-{
-    return __builtin_amdgcn_bitop3_b32(x, y, m, 0x28);
-}
-
-template <int TYPE, int TM, int NG>
+// TM rows x 4*NG columns per thread; KCH = packed 64-bit words of K per chunk, at most;
+// PIPE = operand fragments double-buffered in registers (costs APL*TM + BPL*4*NG VGPRs).
+template <int TYPE, int TM, int NG, int KCH, bool PIPE>
 __global__ __launch_bounds__(kThreads) void conv_popcount(const ConvArgs p)
 {
     constexpr int APL = Planes<TYPE>::A, BPL = Planes<TYPE>::B;
     constexpr int BM = 16 * TM, BN = 64 * NG, TN = 4 * NG;
+    constexpr int kMaxChunkWords = KCH, kMaxQ = 2 * KCH;  // 32-bit k-slices per chunk
     constexpr int A_DWORDS = APL * kMaxQ * BM, B_DWORDS = BPL * kMaxQ * BN;
     constexpr int A_STEP = kThreads / BM;                      // words fetched per pass over the tile rows
     constexpr int B_STEP = kThreads / BN;
@@ -153,12 +197,12 @@ __global__ __launch_bounds__(kThreads) void conv_popcount(const ConvArgs p)
 #pragma unroll
         for (int i = 0; i < A_ITEMS; i++) {
             const int w = a_w0 + i * A_STEP;
-            if (w < kMaxChunkWords) store_item<APL, BM>(la, a_reg[i], w, a_row);
+            if (w < kMaxChunkWords) store_item<APL, BM, kMaxQ>(la, a_reg[i], w, a_row);
         }
 #pragma unroll
         for (int i = 0; i < B_ITEMS; i++) {
             const int w = b_w0 + i * B_STEP;
-            if (w < kMaxChunkWords) store_item<BPL, BN>(lb, b_reg[i], w, b_row);
+            if (w < kMaxChunkWords) store_item<BPL, BN, kMaxQ>(lb, b_reg[i], w, b_row);
         }
     };
 
@@ -217,22 +261,15 @@ __global__ __launch_bounds__(kThreads) void conv_popcount(const ConvArgs p)
 #pragma unroll
         for (int i = 0; i < TM; i++)
 #pragma unroll
-            for (int j = 0; j < TN; j++) {
-                if (TYPE == 0) {
-                    // TAB_GEMM.cu:48-51
-                    const uint32_t both = f.a[1][i] & f.b[1][j];
-                    popcount_acc(nzc[i][j], both);
-                    popcount_acc(acc[i][j], xor_and(f.a[0][i], f.b[0][j], both));
-                } else if (TYPE == 1) {
-                    // TAB_GEMM.cu:81-84; popcount(a1) is summed once per row above
-                    popcount_acc(acc[i][j], xor_and(f.a[0][i], f.b[0][j], f.a[1][i]));
-                } else if (TYPE == 2) {
-                    // TAB_GEMM.cu:113-114
-                    popcount_acc(acc[i][j], xor_and(f.a[0][i], f.b[0][j], f.b[1][j]));
-                } else {
-                    // TAB_GEMM.cu:142
-                    popcount_acc(acc[i][j], f.a[0][i] ^ f.b[0][j]);
-                }
+            for (int j = 0; j < TN; j += 4) {
+                if (TYPE == 0)
+                    tnn_quad(&nzc[i][j], &acc[i][j], f.a[0][i], f.a[1][i], &f.b[0][j], &f.b[1][j]);
+                else if (TYPE == 1)
+                    tbn_quad(&acc[i][j], f.a[0][i], f.a[1][i], &f.b[0][j]);  // popcount(a1) is summed once per row above
+                else if (TYPE == 2)
+                    btn_quad(&acc[i][j], f.a[0][i], &f.b[0][j], &f.b[1][j]);
+                else
+                    bnn_quad(&acc[i][j], f.a[0][i], &f.b[0][j]);
             }
     };
 
@@ -251,20 +288,28 @@ __global__ __launch_bounds__(kThreads) void conv_popcount(const ConvArgs p)
         // work of slice q, so a single wave per SIMD still keeps the VALU busy.  nq is even.
         // The read of slice nq after the last pair stays inside the LDS allocation (one spare
         // slice is reserved) and its value is never used.
-        Frag f0, f1;
-        // drain outstanding scalar loads first: they share the LDS counter and return out of
-        // order, which would force full waits inside the loop
-        __builtin_amdgcn_s_waitcnt(0xc07f);
-        read_frag(f0, la, lb, 0);
-        for (int q = 0; q < nq; q += 2) {
-            read_frag(f1, la, lb, q + 1);
-            __builtin_amdgcn_sched_barrier(0);
-            mac(f0);
-            __builtin_amdgcn_sched_barrier(0);
-            read_frag(f0, la, lb, q + 2);
-            __builtin_amdgcn_sched_barrier(0);
-            mac(f1);
-            __builtin_amdgcn_sched_barrier(0);
+        if (PIPE) {
+            Frag f0, f1;
+            // drain outstanding scalar loads first: they share the LDS counter and return out
+            // of order, which would force full waits inside the loop
+            __builtin_amdgcn_s_waitcnt(0xc07f);
+            read_frag(f0, la, lb, 0);
+            for (int q = 0; q < nq; q += 2) {
+                read_frag(f1, la, lb, q + 1);
+                __builtin_amdgcn_sched_barrier(0);
+                mac(f0);
+                __builtin_amdgcn_sched_barrier(0);
+                read_frag(f0, la, lb, q + 2);
+                __builtin_amdgcn_sched_barrier(0);
+                mac(f1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+            for (int q = 0; q < nq; q++) {
+                Frag f;
+                read_frag(f, la, lb, q);
+                mac(f);
+            }
         }
 
         if (more) stage((chunk + 1) & 1);
@@ -308,39 +353,75 @@ __global__ __launch_bounds__(kThreads) void conv_popcount(const ConvArgs p)
     }
 }
 
-template <int TYPE, int TM, int NG>
+// Extra (unused) dynamic LDS per workgroup that makes the number of resident workgroups per
+// CU - one wave per SIMD each - even: the VALU pairing above only pays off with an even number
+// of waves per SIMD (2 or 4; 3 measured as slow as no pairing at all).
+template <typename Kernel>
+int even_occupancy_lds(Kernel kernel)
+{
+    int dyn = 0;
+    for (; dyn <= 48 * 1024; dyn += 2048) {
+        int blocks = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, kernel, kThreads, dyn) != hipSuccess) {
+            (void)hipGetLastError();
+            return 0;
+        }
+        if (blocks <= 2 || (blocks & 1) == 0) return dyn;
+    }
+    return 0;
+}
+
+template <int TYPE, int TM, int NG, int KCH, bool PIPE = true>
 hipError_t launch_tile(ConvArgs a, hipStream_t stream)
 {
     constexpr int BM = 16 * TM, BN = 64 * NG;
+    static const int dyn_lds = even_occupancy_lds(conv_popcount<TYPE, TM, NG, KCH, PIPE>);
+    // chunk length: at most KCH words, chunks of equal length
+    a.nchunks = (a.G + KCH - 1) / KCH;
+    a.kcw = (a.G + a.nchunks - 1) / a.nchunks;
+    a.nchunks = (a.G + a.kcw - 1) / a.kcw;
     a.tiles_m = (a.M + BM - 1) / BM;
     const long tiles_n = (a.KN + BN - 1) / BN;
     const long blocks = (long)a.tiles_m * tiles_n;
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
-    conv_popcount<TYPE, TM, NG><<<dim3((unsigned)blocks), dim3(kThreads), 0, stream>>>(a);
+    conv_popcount<TYPE, TM, NG, KCH, PIPE><<<dim3((unsigned)blocks), dim3(kThreads), dyn_lds, stream>>>(a);
     return hipGetLastError();
 }
 
 // Tuning hook (not part of the public ABI): forces one tile shape for every launch.
 int g_force_tm = 0, g_force_ng = 0;
 
-// Tile choice: the largest tile that still gives every CU a few workgroups; small layers
-// fall back to smaller tiles so that the 256 CUs are not left idle.
+// Tile shapes.  Every shape keeps <= 128 VGPRs, i.e. 4 workgroups (4 waves per SIMD) per CU;
+// measured on N=256 28x28x512->512 3x3, shapes with 128 accumulators at 2 waves per SIMD were
+// 15-25 % slower than these.  `Big` is the 128-row tile of each type: 128x128 where one
+// accumulator per output suffices, 128x64 for TNN (two counts per output); fragments are
+// register double-buffered only where that still fits 128 VGPRs (BNN).
+template <int TYPE>
+hipError_t launch_big(const ConvArgs &a, hipStream_t stream)
+{
+    if (TYPE == 0) return launch_tile<TYPE, 8, 1, 4, false>(a, stream);
+    if (TYPE == 3) return launch_tile<TYPE, 8, 2, 4, true>(a, stream);
+    return launch_tile<TYPE, 8, 2, 4, false>(a, stream);
+}
+
+// Tile choice: the largest tile that still gives every CU at least two workgroups; small
+// layers fall back to smaller tiles so that the 256 CUs are not left idle.
 template <int TYPE>
 hipError_t launch_type(const ConvArgs &a, hipStream_t stream)
 {
+    constexpr int BIG_BN = (TYPE == 0) ? 64 : 128;
     if (g_force_tm) {
-        const int ng = (TYPE == 0) ? 1 : g_force_ng;
-        if (g_force_tm == 8 && ng == 2) return launch_tile<TYPE, 8, (TYPE == 0 ? 1 : 2)>(a, stream);
-        if (g_force_tm == 8) return launch_tile<TYPE, 8, 1>(a, stream);
-        if (g_force_tm == 4) return launch_tile<TYPE, 4, 1>(a, stream);
-        return launch_tile<TYPE, 2, 1>(a, stream);
+        if (g_force_tm == 8 && g_force_ng == 2) return launch_big<TYPE>(a, stream);
+        if (g_force_tm == 8) return launch_tile<TYPE, 8, 1, 4, false>(a, stream);
+        if (g_force_tm == 4) return launch_tile<TYPE, 4, 1, 8, true>(a, stream);
+        return launch_tile<TYPE, 2, 1, 8, true>(a, stream);
     }
-    const long want = 2 * 256;  // at least two workgroups per CU
+    const long want = 2 * 256;
     auto tiles = [&](int bm, int bn) { return (long)((a.M + bm - 1) / bm) * ((a.KN + bn - 1) / bn); };
-    if (TYPE != 0 && a.KN > 64 && tiles(128, 128) >= want) return launch_tile<TYPE, 8, (TYPE == 0 ? 1 : 2)>(a, stream);
-    if (tiles(128, 64) >= want) return launch_tile<TYPE, 8, 1>(a, stream);
-    if (tiles(64, 64) >= want) return launch_tile<TYPE, 4, 1>(a, stream);
-    return launch_tile<TYPE, 2, 1>(a, stream);
+    if (a.KN > BIG_BN / 2 && tiles(128, BIG_BN) >= want) return launch_big<TYPE>(a, stream);
+    if (tiles(128, 64) >= want) return launch_tile<TYPE, 8, 1, 4, false>(a, stream);
+    if (tiles(64, 64) >= want) return launch_tile<TYPE, 4, 1, 8, true>(a, stream);
+    return launch_tile<TYPE, 2, 1, 8, true>(a, stream);
 }
 
 }  // namespace
@@ -353,16 +434,11 @@ void force_conv_tile(int tm, int ng)
 
 hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream)
 {
-    ConvArgs a = args;
-    // chunk length: at most kMaxChunkWords, and such that the chunks are of equal length
-    a.nchunks = (a.G + kMaxChunkWords - 1) / kMaxChunkWords;
-    a.kcw = (a.G + a.nchunks - 1) / a.nchunks;
-    a.nchunks = (a.G + a.kcw - 1) / a.kcw;
     switch (type) {
-    case 0: return launch_type<0>(a, stream);
-    case 1: return launch_type<1>(a, stream);
-    case 2: return launch_type<2>(a, stream);
-    case 3: return launch_type<3>(a, stream);
+    case 0: return launch_type<0>(args, stream);
+    case 1: return launch_type<1>(args, stream);
+    case 2: return launch_type<2>(args, stream);
+    case 3: return launch_type<3>(args, stream);
     default: return hipErrorInvalidValue;
     }
 }
