@@ -326,13 +326,30 @@ def main():
         del xq
         result["quantize"] = {"shape": "256x56x56x256 fp32", "bound": "hbm", "peak_GBps": HBM_PEAK_GBS, **quant}
 
+        # ---- the same ResNet-18 layer set at N=256 (kernels long enough not to be launch-bound)
+        rn_ops, rn_ms, rn_layers = 0, 0.0, []
+        for i, l in enumerate(RESNET18_LAYERS):
+            L = Layer(tab, torch, 3, 256, l, seed=i, on_device=True)
+            k_ms = graph_time_ms(torch, L.conv_kernel_only, 5, replays=4)
+            c_ms = graph_time_ms(torch, L.conv2d, 5, replays=4)
+            rn_ops += L.ops
+            rn_ms += k_ms
+            rn_layers.append({"layer": layer_name(256, l), "conv_kernel_us": round(k_ms * 1e3, 1),
+                              "call_us": round(c_ms * 1e3, 1), "conv_kernel_tops": round(L.ops / k_ms / 1e9, 1),
+                              "frac_valu_peak": round(L.ops / k_ms / 1e9 / valu_peak_tops(3), 4)})
+            del L
+        result["resnet18_bnn_N256"] = {"conv_kernel_tops": round(rn_ops / rn_ms / 1e9, 1),
+                                       "frac_valu_peak": round(rn_ops / rn_ms / 1e9 / valu_peak_tops(3), 4),
+                                       "frac_of_planning_peak": round(rn_ops / rn_ms / 1e9 / planning_peak_tops(3), 4),
+                                       "layers": rn_layers}
+
         # ---- the largest sweep point, all four types (conv kernel only) --------------------
         big = (28, 28, 512, 512, 3, 3, 1, 1, 1, 1)
         sweep = {}
         for type in range(4):
             L = Layer(tab, torch, type, 256, big, seed=7, relu=(type == 1), on_device=True)
-            k_ms = event_time_ms(torch, L.conv_kernel_only, 5, warmup=2)
-            call_ms = median_call_ms(torch, L.conv2d, 5, warmup=1)
+            k_ms = graph_time_ms(torch, L.conv_kernel_only, 5, replays=4)
+            call_ms = graph_time_ms(torch, L.conv2d, 3, replays=3)
             sweep[TYPE_NAMES[type]] = {"conv_kernel_ms": round(k_ms, 3), "call_ms": round(call_ms, 3),
                                        "conv_kernel_tops": round(L.ops / k_ms / 1e9, 1),
                                        "valu_peak_tops": round(valu_peak_tops(type), 1),

@@ -18,7 +18,6 @@
 namespace tab {
 namespace {
 
-constexpr int kThreads = 256;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -119,12 +118,15 @@ __device__ __forceinline__ void popcount_acc(int &acc, uint32_t x)
 }
 
 // TM rows x 4*NG columns per thread; KCH = packed 64-bit words of K per chunk, at most;
-// PIPE = operand fragments double-buffered in registers (costs APL*TM + BPL*4*NG VGPRs).
-template <int TYPE, int TM, int NG, int KCH, bool PIPE>
-__global__ __launch_bounds__(kThreads) void conv_popcount(const ConvArgs p)
+// PIPE = operand fragments double-buffered in registers (costs APL*TM + BPL*4*NG VGPRs);
+// NT = threads per workgroup: 256 (one wave per SIMD) or 512 (two waves per SIMD, so that the
+// number of waves per SIMD is even whatever the number of resident workgroups).
+template <int TYPE, int TM, int NG, int KCH, bool PIPE, int NT>
+__global__ __launch_bounds__(NT) void conv_popcount(const ConvArgs p)
 {
+    constexpr int kThreads = NT;
     constexpr int APL = Planes<TYPE>::A, BPL = Planes<TYPE>::B;
-    constexpr int BM = 16 * TM, BN = 64 * NG, TN = 4 * NG;
+    constexpr int BM = (NT / 16) * TM, BN = 64 * NG, TN = 4 * NG;
     constexpr int kMaxChunkWords = KCH, kMaxQ = 2 * KCH;  // 32-bit k-slices per chunk
     constexpr int A_DWORDS = APL * kMaxQ * BM, B_DWORDS = BPL * kMaxQ * BN;
     constexpr int A_STEP = kThreads / BM;                      // words fetched per pass over the tile rows
@@ -356,26 +358,31 @@ __global__ __launch_bounds__(kThreads) void conv_popcount(const ConvArgs p)
 // Extra (unused) dynamic LDS per workgroup that makes the number of resident workgroups per
 // CU - one wave per SIMD each - even: the VALU pairing above only pays off with an even number
 // of waves per SIMD (2 or 4; 3 measured as slow as no pairing at all).
+struct Occupancy {
+    int dyn_lds;        // bytes of padding LDS per workgroup
+    int blocks_per_cu;  // resident workgroups per CU with that padding (0 = unknown)
+};
+
 template <typename Kernel>
-int even_occupancy_lds(Kernel kernel)
+Occupancy even_occupancy(Kernel kernel, int kThreads)
 {
-    int dyn = 0;
-    for (; dyn <= 48 * 1024; dyn += 2048) {
+    if (kThreads == 512) return {0, 0};  // two waves per SIMD per workgroup: always even
+    for (int dyn = 0; dyn <= 48 * 1024; dyn += 2048) {
         int blocks = 0;
         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, kernel, kThreads, dyn) != hipSuccess) {
             (void)hipGetLastError();
-            return 0;
+            return {0, 0};
         }
-        if (blocks <= 2 || (blocks & 1) == 0) return dyn;
+        if (blocks <= 2 || (blocks & 1) == 0) return {dyn, blocks};
     }
-    return 0;
+    return {0, 0};
 }
 
-template <int TYPE, int TM, int NG, int KCH, bool PIPE = true>
+template <int TYPE, int TM, int NG, int KCH, bool PIPE = true, int NT = 256>
 hipError_t launch_tile(ConvArgs a, hipStream_t stream)
 {
-    constexpr int BM = 16 * TM, BN = 64 * NG;
-    static const int dyn_lds = even_occupancy_lds(conv_popcount<TYPE, TM, NG, KCH, PIPE>);
+    constexpr int BM = (NT / 16) * TM, BN = 64 * NG;
+    static const Occupancy occ = even_occupancy(conv_popcount<TYPE, TM, NG, KCH, PIPE, NT>, NT);
     // chunk length: at most KCH words, chunks of equal length
     a.nchunks = (a.G + KCH - 1) / KCH;
     a.kcw = (a.G + a.nchunks - 1) / a.nchunks;
@@ -384,43 +391,46 @@ hipError_t launch_tile(ConvArgs a, hipStream_t stream)
     const long tiles_n = (a.KN + BN - 1) / BN;
     const long blocks = (long)a.tiles_m * tiles_n;
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
-    conv_popcount<TYPE, TM, NG, KCH, PIPE><<<dim3((unsigned)blocks), dim3(kThreads), dyn_lds, stream>>>(a);
+    conv_popcount<TYPE, TM, NG, KCH, PIPE, NT><<<dim3((unsigned)blocks), dim3(NT), occ.dyn_lds, stream>>>(a);
     return hipGetLastError();
 }
 
 // Tuning hook (not part of the public ABI): forces one tile shape for every launch.
 int g_force_tm = 0, g_force_ng = 0;
 
-// Tile shapes.  Every shape keeps <= 128 VGPRs, i.e. 4 workgroups (4 waves per SIMD) per CU;
-// measured on N=256 28x28x512->512 3x3, shapes with 128 accumulators at 2 waves per SIMD were
-// 15-25 % slower than these.  `Big` is the 128-row tile of each type: 128x128 where one
-// accumulator per output suffices, 128x64 for TNN (two counts per output); fragments are
-// register double-buffered only where that still fits 128 VGPRs (BNN).
+// Tile shapes.  Every shape keeps <= 128 VGPRs, i.e. at least 4 workgroups (4 waves per SIMD)
+// per CU; shapes with 128 accumulators at 2 waves per SIMD and 512-thread workgroups were
+// measured 10-25 % slower.  Three shapes are used:
+//   big    128x128 (128x64 for TNN, which keeps two counts per output), chunks of 4 words;
+//          fragments register double-buffered only where that still fits 128 VGPRs (BNN)
+//   medium 64x64, chunks of 4 words, double-buffered fragments, 8 workgroups per CU
+//   small  32x64, chunks of 8 words
+// Measured over the ResNet-18 / sweep shapes at N = 32..256: the medium tile wins everywhere
+// except on the very largest launches (>= 3 rounds of big tiles over the whole chip), and the
+// small tile wins once even medium tiles give the CUs fewer than two workgroups each.
 template <int TYPE>
 hipError_t launch_big(const ConvArgs &a, hipStream_t stream)
 {
-    if (TYPE == 0) return launch_tile<TYPE, 8, 1, 4, false>(a, stream);
-    if (TYPE == 3) return launch_tile<TYPE, 8, 2, 4, true>(a, stream);
-    return launch_tile<TYPE, 8, 2, 4, false>(a, stream);
+    if constexpr (TYPE == 0)
+        return launch_tile<TYPE, 8, 1, 4, false>(a, stream);
+    else if constexpr (TYPE == 3)
+        return launch_tile<TYPE, 8, 2, 4, true>(a, stream);
+    else
+        return launch_tile<TYPE, 8, 2, 4, false>(a, stream);
 }
 
-// Tile choice: the largest tile that still gives every CU at least two workgroups; small
-// layers fall back to smaller tiles so that the 256 CUs are not left idle.
 template <int TYPE>
 hipError_t launch_type(const ConvArgs &a, hipStream_t stream)
 {
     constexpr int BIG_BN = (TYPE == 0) ? 64 : 128;
     if (g_force_tm) {
-        if (g_force_tm == 8 && g_force_ng == 2) return launch_big<TYPE>(a, stream);
-        if (g_force_tm == 8) return launch_tile<TYPE, 8, 1, 4, false>(a, stream);
-        if (g_force_tm == 4) return launch_tile<TYPE, 4, 1, 8, true>(a, stream);
+        if (g_force_tm == 8) return launch_big<TYPE>(a, stream);
+        if (g_force_tm == 4) return launch_tile<TYPE, 4, 1, 4, true>(a, stream);
         return launch_tile<TYPE, 2, 1, 8, true>(a, stream);
     }
-    const long want = 2 * 256;
     auto tiles = [&](int bm, int bn) { return (long)((a.M + bm - 1) / bm) * ((a.KN + bn - 1) / bn); };
-    if (a.KN > BIG_BN / 2 && tiles(128, BIG_BN) >= want) return launch_big<TYPE>(a, stream);
-    if (tiles(128, 64) >= want) return launch_tile<TYPE, 8, 1, 4, false>(a, stream);
-    if (tiles(64, 64) >= want) return launch_tile<TYPE, 4, 1, 8, true>(a, stream);
+    if (a.KN > BIG_BN / 2 && tiles(128, BIG_BN) >= 3072) return launch_big<TYPE>(a, stream);
+    if (tiles(64, 64) >= 512) return launch_tile<TYPE, 4, 1, 4, true>(a, stream);
     return launch_tile<TYPE, 2, 1, 8, true>(a, stream);
 }
 
