@@ -323,6 +323,9 @@ def main():
             quant[f"bitwidth{bitwidth}"] = {"us": round(ms * 1e3, 1), "GBps": round(nbytes / ms / 1e6, 1),
                                             "frac_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
                                             "bytes": nbytes}
+        ms = event_time_ms(torch, lambda: tab.Threshold(xq, qN, 0.7), 20)
+        quant["threshold_abs_mean"] = {"us": round(ms * 1e3, 1), "GBps": round(4 * qN * qH * qW * qC / ms / 1e6, 1),
+                                       "frac_hbm_peak": round(4 * qN * qH * qW * qC / ms / 1e6 / HBM_PEAK_GBS, 4)}
         del xq
         result["quantize"] = {"shape": "256x56x56x256 fp32", "bound": "hbm", "peak_GBps": HBM_PEAK_GBS, **quant}
 

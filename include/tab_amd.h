@@ -63,6 +63,19 @@ int tab_quantize(const float *dev_X, const float *dev_ths, int bitwidth, int N, 
                  int C, int64_t *dev_QX, int32_t *dev_BTN, void *stream);
 
 /*
+ * Per-item threshold ths[n] = scale * mean(|X[n]|) over per_item consecutive fp32 values: the
+ * step before Quantize/Conv2d, which the reference leaves to the caller (README.md:45,
+ * "threshold values of each filter or each input image"; the usual ternary rule is
+ * scale = 0.7).  It has no counterpart function in the reference.  Floating point: a
+ * fixed-order fp32 tree per slice and an fp64 sum of the slices, reproducible from run to
+ * run; agrees with an fp64 reference to a relative 1e-5.
+ *   workspace: tab_threshold_workspace_bytes(N, per_item) bytes of device scratch.
+ */
+size_t tab_threshold_workspace_bytes(int N, long per_item);
+int tab_threshold(const float *dev_X, int N, long per_item, float scale, float *dev_ths,
+                  void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * Bytes of device scratch tab_conv2d needs for the packed activation
  * (the reference cudaMallocs pad_a/img_a per call, TAB_GEMM.cu:391-397).  0 on bad arguments.
  */

@@ -79,6 +79,25 @@ def Quantize(X, thresholds, bitwidth, N, H, W, C):
     return [QX, BTN]
 
 
+def Threshold(X, N, scale=0.7):
+    """ths[n] = scale * mean(|X[n]|) per item (image or filter), fp32 (N,), computed on the
+    device in one pass: the threshold rule the reference leaves to the caller (README.md:45).
+    Reproducible from run to run; within 1e-5 relative of an fp64 reference."""
+    _check_input(X, "X")
+    _check_dtype(X, torch.float32, "X")
+    N = int(N)
+    if N < 1 or X.numel() % N != 0 or X.numel() == 0:
+        raise RuntimeError(f"X has {X.numel()} elements, not a positive multiple of N = {N}")
+    per_item = X.numel() // N
+    with torch.cuda.device(X.device):
+        ths = torch.empty((N,), dtype=torch.float32, device=X.device)
+        ws_bytes = _lib.tab_threshold_workspace_bytes(N, per_item)
+        ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=X.device)
+        _capi.check(_lib, _lib.tab_threshold(X.data_ptr(), N, per_item, float(scale), ths.data_ptr(),
+                                             ws.data_ptr(), ws_bytes, _stream()))
+    return ths
+
+
 def _conv_checks(QW, btn, type, N, H, W, C, KN, KH, KW, pad1, pad2, stride1, stride2):
     if type not in (0, 1, 2, 3):
         raise RuntimeError(f"type must be 0 (TNN), 1 (TBN), 2 (BTN) or 3 (BNN), got {type}")
@@ -153,5 +172,5 @@ def Conv2dPacked(QX, QW, btn, type, padding1, padding2, stride1, stride2, N, H, 
 TAB_Quantize = Quantize
 TAB_Conv2d = Conv2d
 
-__all__ = ["Quantize", "Conv2d", "Conv2dPacked", "TAB_Quantize", "TAB_Conv2d", "TabError",
+__all__ = ["Quantize", "Conv2d", "Conv2dPacked", "Threshold", "TAB_Quantize", "TAB_Conv2d", "TabError",
            "packed_channels", "out_shape", "version", "TNN", "TBN", "BTN", "BNN"]

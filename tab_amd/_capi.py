@@ -18,6 +18,8 @@ SIGNATURES = {
     "tab_packed_channels": (_int, [_int]),
     "tab_out_extent": (_int, [_int] * 4),
     "tab_quantize": (_int, [_vp, _vp, _int, _int, _int, _int, _int, _vp, _vp, _vp]),
+    "tab_threshold_workspace_bytes": (_sz, [_int, ctypes.c_long]),
+    "tab_threshold": (_int, [_vp, _int, ctypes.c_long, ctypes.c_float, _vp, _vp, _sz, _vp]),
     "tab_conv2d_workspace_bytes": (_sz, [_int] * 5),
     "tab_conv2d": (_int, [_vp] * 4 + [_int] * 12 + [_vp, _vp, _sz, _vp]),
     "tab_conv2d_packed": (_int, [_vp] * 3 + [_int] * 12 + [_vp, _vp]),

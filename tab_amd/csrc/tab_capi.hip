@@ -99,6 +99,26 @@ int tab_quantize(const float *dev_X, const float *dev_ths, int bitwidth, int N, 
     return TAB_OK;
 }
 
+size_t tab_threshold_workspace_bytes(int N, long per_item)
+{
+    if (N < 1 || per_item < 1) return 0;
+    return (size_t)N * tab::threshold_splits(N, per_item) * sizeof(float);
+}
+
+int tab_threshold(const float *dev_X, int N, long per_item, float scale, float *dev_ths, void *workspace,
+                  size_t workspace_bytes, void *stream)
+{
+    if (N < 1 || per_item < 1) return fail(TAB_ERR_BAD_ARGUMENT, "N and per_item must be positive");
+    if (!dev_X || !dev_ths) return fail(TAB_ERR_BAD_ARGUMENT, "null device pointer");
+    const size_t need = tab_threshold_workspace_bytes(N, per_item);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace % 4))
+        return fail(TAB_ERR_WORKSPACE, "workspace must hold %zu bytes (got %zu)", need, workspace_bytes);
+    hipError_t e = tab::launch_threshold(dev_X, N, per_item, scale, dev_ths, static_cast<float *>(workspace),
+                                         static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return device_fail(e, "threshold launch");
+    return TAB_OK;
+}
+
 size_t tab_conv2d_workspace_bytes(int type, int N, int H, int W, int C)
 {
     if (type < 0 || type > 3 || N < 1 || H < 1 || W < 1 || C < 1) return 0;

@@ -52,6 +52,12 @@ hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream);
 hipError_t launch_quantize(const float *x, const float *ths, int bitwidth, long pixels_per_item,
                            long items, int C, uint64_t *qx, int32_t *btn, hipStream_t stream);
 
+// ths[n] = scale * mean|x[n]| over per_item elements; `partial` holds items * threshold_splits()
+// floats of scratch.
+int threshold_splits(long items, long per_item);
+hipError_t launch_threshold(const float *x, long items, long per_item, float scale, float *ths, float *partial,
+                            hipStream_t stream);
+
 void force_conv_tile(int tm, int ng);  // tuning hook: 0,0 restores the automatic choice
 
 }  // namespace tab

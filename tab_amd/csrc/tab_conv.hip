@@ -18,6 +18,7 @@
 namespace tab {
 namespace {
 
+constexpr int kThreads = 256;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -118,15 +119,13 @@ __device__ __forceinline__ void popcount_acc(int &acc, uint32_t x)
 }
 
 // TM rows x 4*NG columns per thread; KCH = packed 64-bit words of K per chunk, at most;
-// PIPE = operand fragments double-buffered in registers (costs APL*TM + BPL*4*NG VGPRs);
-// NT = threads per workgroup: 256 (one wave per SIMD) or 512 (two waves per SIMD, so that the
-// number of waves per SIMD is even whatever the number of resident workgroups).
-template <int TYPE, int TM, int NG, int KCH, bool PIPE, int NT>
-__global__ __launch_bounds__(NT) void conv_popcount(const ConvArgs p)
+// PIPE = operand fragments double-buffered in registers (costs APL*TM + BPL*4*NG VGPRs).
+// 256 threads: one wave per SIMD (512-thread workgroups were measured slightly slower).
+template <int TYPE, int TM, int NG, int KCH, bool PIPE>
+__global__ __launch_bounds__(kThreads) void conv_popcount(const ConvArgs p)
 {
-    constexpr int kThreads = NT;
     constexpr int APL = Planes<TYPE>::A, BPL = Planes<TYPE>::B;
-    constexpr int BM = (NT / 16) * TM, BN = 64 * NG, TN = 4 * NG;
+    constexpr int BM = 16 * TM, BN = 64 * NG, TN = 4 * NG;
     constexpr int kMaxChunkWords = KCH, kMaxQ = 2 * KCH;  // 32-bit k-slices per chunk
     constexpr int A_DWORDS = APL * kMaxQ * BM, B_DWORDS = BPL * kMaxQ * BN;
     constexpr int A_STEP = kThreads / BM;                      // words fetched per pass over the tile rows
@@ -364,9 +363,8 @@ struct Occupancy {
 };
 
 template <typename Kernel>
-Occupancy even_occupancy(Kernel kernel, int kThreads)
+Occupancy even_occupancy(Kernel kernel)
 {
-    if (kThreads == 512) return {0, 0};  // two waves per SIMD per workgroup: always even
     for (int dyn = 0; dyn <= 48 * 1024; dyn += 2048) {
         int blocks = 0;
         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, kernel, kThreads, dyn) != hipSuccess) {
@@ -378,11 +376,11 @@ Occupancy even_occupancy(Kernel kernel, int kThreads)
     return {0, 0};
 }
 
-template <int TYPE, int TM, int NG, int KCH, bool PIPE = true, int NT = 256>
+template <int TYPE, int TM, int NG, int KCH, bool PIPE = true>
 hipError_t launch_tile(ConvArgs a, hipStream_t stream)
 {
-    constexpr int BM = (NT / 16) * TM, BN = 64 * NG;
-    static const Occupancy occ = even_occupancy(conv_popcount<TYPE, TM, NG, KCH, PIPE, NT>, NT);
+    constexpr int BM = 16 * TM, BN = 64 * NG;
+    static const Occupancy occ = even_occupancy(conv_popcount<TYPE, TM, NG, KCH, PIPE>);
     // chunk length: at most KCH words, chunks of equal length
     a.nchunks = (a.G + KCH - 1) / KCH;
     a.kcw = (a.G + a.nchunks - 1) / a.nchunks;
@@ -391,7 +389,7 @@ hipError_t launch_tile(ConvArgs a, hipStream_t stream)
     const long tiles_n = (a.KN + BN - 1) / BN;
     const long blocks = (long)a.tiles_m * tiles_n;
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
-    conv_popcount<TYPE, TM, NG, KCH, PIPE, NT><<<dim3((unsigned)blocks), dim3(NT), occ.dyn_lds, stream>>>(a);
+    conv_popcount<TYPE, TM, NG, KCH, PIPE><<<dim3((unsigned)blocks), dim3(kThreads), occ.dyn_lds, stream>>>(a);
     return hipGetLastError();
 }
 

@@ -17,6 +17,8 @@ constexpr int kLoadsPerLane = 8;                // float4 loads in flight per la
 constexpr int kRowsPerWave = 4 * kLoadsPerLane; // each wave-wide float4 load covers 4 rows
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef uint32_t uintx4 __attribute__((ext_vector_type(4)));
+typedef uint32_t uintx2 __attribute__((ext_vector_type(2)));
 
 // OR over the 8 lanes of each half of a 16-lane DPP row; every lane gets the result.
 __device__ __forceinline__ uint32_t or_reduce8(uint32_t v)
@@ -25,6 +27,12 @@ __device__ __forceinline__ uint32_t or_reduce8(uint32_t v)
     v |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
     v |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xF, 0xF, true);  // row_half_mirror
     return v;
+}
+
+// value of the lane 8 positions further round the 16-lane DPP row (row_ror:8)
+__device__ __forceinline__ uint32_t rotate_row8(uint32_t v)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x128, 0xF, 0xF, true);
 }
 
 __device__ __forceinline__ int wave_sum(int v)
@@ -95,16 +103,18 @@ __global__ __launch_bounds__(kThreads) void quantize_rows64(const floatx4 *__res
         uint32_t sign, nz;
         compare4<BITS>(v[u], t, sign, nz);
         const int shift = 4 * (l & 7);
-        const uint32_t sign_word = or_reduce8(sign << shift);
+        // after the reduction lanes 0-7 of the row hold the low half, lanes 8-15 the high half;
+        // a rotate by 8 within the row hands lane 0 the other half, and lane 0 stores the whole
+        // element (8 or 16 bytes) at once
+        const uint32_t sign_half = or_reduce8(sign << shift);
+        const uint32_t sign_other = rotate_row8(sign_half);
         if (BITS == 2) {
-            const uint32_t nz_word = or_reduce8(nz << shift);
-            // dword (r*2 + plane)*2 + half; lanes 0/1 of each half-row store plane 0/1
-            if (r < rows && (l & 7) < 2) {
-                const int plane = l & 1, half = l >> 3;
-                q[(r * 2 + plane) * 2 + half] = plane ? nz_word : sign_word;
-            }
+            const uint32_t nz_half = or_reduce8(nz << shift);
+            const uint32_t nz_other = rotate_row8(nz_half);
+            if (r < rows && l == 0)
+                *reinterpret_cast<uintx4 *>(q + r * 4) = uintx4{sign_half, sign_other, nz_half, nz_other};
         } else {
-            if (r < rows && (l & 7) == 0) q[r * 2 + (l >> 3)] = sign_word;
+            if (r < rows && l == 0) *reinterpret_cast<uintx2 *>(q + r * 2) = uintx2{sign_half, sign_other};
         }
     }
 }
@@ -185,7 +195,75 @@ __global__ __launch_bounds__(kThreads) void btn_popcount(const ulonglong2 *__res
     }
 }
 
+// ---- thresholds: ths[n] = scale * mean(|x[n]|) ------------------------------------------------
+// The step right before Quantize in the reference's demo flow (the caller computes it in
+// torch).  Two fixed-order stages so that the result does not depend on scheduling: `splits`
+// workgroups per item each reduce a contiguous slice to one fp32 partial (per-thread serial
+// sums of float4, then a tree over lanes and waves), then one thread per item adds the
+// partials in index order in fp64.
+__global__ __launch_bounds__(kThreads) void abs_sum_partial(const float *__restrict__ x, float *__restrict__ partial,
+                                                            long per_item, int splits)
+{
+    __shared__ float wave_part[kWavesPerBlock];
+    const long item = blockIdx.x / splits;
+    const int split = blockIdx.x % splits;
+    const long slice = ((per_item + splits - 1) / splits + 3) & ~3L;  // multiple of 4 elements
+    const long begin = split * slice;
+    long end = begin + slice;
+    if (end > per_item) end = per_item;
+    const float *src = x + item * per_item;
+    float sum = 0.f;
+    if (((uintptr_t)(src + begin) & 15) == 0) {
+        const long n4 = begin < end ? (end - begin) / 4 : 0;
+        const floatx4 *src4 = reinterpret_cast<const floatx4 *>(src + begin);
+        for (long i = threadIdx.x; i < n4; i += kThreads) {
+            const floatx4 v = __builtin_nontemporal_load(&src4[i]);
+            sum += (__builtin_fabsf(v[0]) + __builtin_fabsf(v[1])) + (__builtin_fabsf(v[2]) + __builtin_fabsf(v[3]));
+        }
+        for (long i = begin + n4 * 4 + threadIdx.x; i < end; i += kThreads) sum += __builtin_fabsf(src[i]);
+    } else {
+        for (long i = begin + threadIdx.x; i < end; i += kThreads) sum += __builtin_fabsf(src[i]);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_down(sum, off, 64);
+    if ((threadIdx.x & 63) == 0) wave_part[threadIdx.x >> 6] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float total = 0.f;
+#pragma unroll
+        for (int w = 0; w < kWavesPerBlock; w++) total += wave_part[w];
+        partial[blockIdx.x] = total;
+    }
+}
+
+__global__ void abs_mean_finish(const float *__restrict__ partial, float *__restrict__ ths, long items, int splits,
+                                double scale_over_count)
+{
+    const long n = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (n >= items) return;
+    double total = 0.0;
+    for (int s = 0; s < splits; s++) total += (double)partial[n * splits + s];
+    ths[n] = (float)(total * scale_over_count);
+}
+
 }  // namespace
+
+int threshold_splits(long items, long per_item)
+{
+    int splits = 1;
+    while (splits < 1024 && items * splits < 2048 && per_item / (splits * 2) >= 8L * kThreads) splits *= 2;
+    return splits;
+}
+
+hipError_t launch_threshold(const float *x, long items, long per_item, float scale, float *ths, float *partial,
+                            hipStream_t stream)
+{
+    const int splits = threshold_splits(items, per_item);
+    abs_sum_partial<<<dim3((unsigned)(items * splits)), dim3(kThreads), 0, stream>>>(x, partial, per_item, splits);
+    abs_mean_finish<<<dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream>>>(partial, ths, items, splits,
+                                                                                   (double)scale / (double)per_item);
+    return hipGetLastError();
+}
 
 // x: fp32 [items][pixels_per_item][C]; qx: [items*pixels_per_item][PC][bitwidth];
 // btn: [items] or nullptr (then no counts are produced).
@@ -198,7 +276,7 @@ hipError_t launch_quantize(const float *x, const float *ths, int bitwidth, long 
     // very long items are split over several workgroups for the btn pass
     int splits = 1;
     if (btn && bitwidth == 2 && items < 512) {
-        while (splits < 64 && items * splits < 512 && words_per_item / (splits * 2) >= 16 * kThreads) splits *= 2;
+        while (splits < 64 && items * splits < 512 && words_per_item / (splits * 2) >= 2 * kThreads) splits *= 2;
     }
     if (btn && (bitwidth != 2 || splits > 1)) {
         // zeros for 1-bit (TAB_GEMM.cu:283); a kernel rather than a memset node so that the
