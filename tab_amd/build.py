@@ -6,7 +6,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libtab_amd.so")
-SOURCES = ["tab_capi.hip", "tab_conv.hip", "tab_quantize.hip"]
+SOURCES = ["tab_capi.hip", "tab_conv.hip", "tab_conv_mfma.hip", "tab_quantize.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -packed-fp32-ops: keep the compiler from forming packed-FP32 VALU ops from float code.
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall",

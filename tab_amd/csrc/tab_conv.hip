@@ -13,54 +13,12 @@
 // one k-slice with 128-bit LDS reads (A reads broadcast over the 16 tx lanes, B reads are
 // 256 B contiguous per 16 lanes).  The inner loop is pure VALU: XOR/AND + v_bcnt_u32_b32
 // with the count accumulated in the instruction's addend.
-#include "tab_common.h"
+#include "tab_conv_stage.h"
 
 namespace tab {
 namespace {
 
-constexpr int kThreads = 256;
-
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-
-template <int TYPE> struct Planes {
-    static constexpr int A = (TYPE == 0 || TYPE == 1) ? 2 : 1;  // activation planes (TAB_GEMM.cu:367-372)
-    static constexpr int B = (TYPE == 0 || TYPE == 2) ? 2 : 1;  // weight planes (TAB_GEMM.cu:374-379)
-};
-
-// Fetch of one packed word (all planes) of one row of an operand, kept in registers
-// between the global load and the LDS store.
-template <int PL> struct Item {
-    uint32_t d[2 * PL];  // plane-major in memory: [plane][half] as 64-bit words
-};
-
-template <int PL>
-__device__ __forceinline__ Item<PL> load_item(const uint64_t *p, bool valid)
-{
-    Item<PL> it;
-    if (PL == 2) {
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (valid) v = *reinterpret_cast<const u32x4 *>(p);
-        it.d[0] = v[0]; it.d[1] = v[1]; it.d[2] = v[2]; it.d[3] = v[3];
-    } else {
-        u32x2 v = {0u, 0u};
-        if (valid) v = *reinterpret_cast<const u32x2 *>(p);
-        it.d[0] = v[0]; it.d[1] = v[1];
-    }
-    return it;
-}
-
-// LDS placement: dword index ((plane*Q + q) * ROWS + row), Q = 32-bit k-slices per chunk
-template <int PL, int ROWS, int Q>
-__device__ __forceinline__ void store_item(uint32_t *lds, const Item<PL> &it, int word, int row)
-{
-#pragma unroll
-    for (int pl = 0; pl < PL; pl++)
-#pragma unroll
-        for (int half = 0; half < 2; half++)
-            lds[((pl * Q) + 2 * word + half) * ROWS + row] = it.d[pl * 2 + half];
-}
+constexpr int kThreads = kConvThreads;
 
 // Inner-loop primitives.  Measured on MI355X (tab_amd/lib/valu_peak and register-level probes):
 // a SIMD issues v_xor/v_and/v_bitop3 in 2 cycles and v_bcnt_u32_b32 in 4, but only when one
@@ -126,13 +84,8 @@ __global__ __launch_bounds__(kThreads) void conv_popcount(const ConvArgs p)
 {
     constexpr int APL = Planes<TYPE>::A, BPL = Planes<TYPE>::B;
     constexpr int BM = 16 * TM, BN = 64 * NG, TN = 4 * NG;
-    constexpr int kMaxChunkWords = KCH, kMaxQ = 2 * KCH;  // 32-bit k-slices per chunk
-    constexpr int A_DWORDS = APL * kMaxQ * BM, B_DWORDS = BPL * kMaxQ * BN;
-    constexpr int A_STEP = kThreads / BM;                      // words fetched per pass over the tile rows
-    constexpr int B_STEP = kThreads / BN;
-    constexpr int A_ITEMS = (kMaxChunkWords + A_STEP - 1) / A_STEP;
-    constexpr int B_ITEMS = (kMaxChunkWords + B_STEP - 1) / B_STEP;
-    static_assert(kThreads % BM == 0 && kThreads % BN == 0, "tile rows must divide the workgroup");
+    using Stager = TileStager<TYPE, BM, BN, KCH>;
+    constexpr int kMaxQ = Stager::Q, A_DWORDS = Stager::A_DWORDS, B_DWORDS = Stager::B_DWORDS;
     static_assert(TM % 4 == 0 || TM == 2, "TM is read with 64- or 128-bit LDS loads");
 
     // + one spare k-slice of the wider operand: the pipelined loop reads one slice ahead
@@ -144,68 +97,8 @@ __global__ __launch_bounds__(kThreads) void conv_popcount(const ConvArgs p)
     const int tile_m = blockIdx.x % p.tiles_m, tile_n = blockIdx.x / p.tiles_m;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
-    // ---- staging roles -------------------------------------------------------------------
-    // A: thread fetches words (a_w0 + i*A_STEP) of output pixel m0 + a_row
-    const int a_row = tid % BM, a_w0 = tid / BM;
-    const int a_m = m0 + a_row;
-    const bool a_live = a_m < p.M;
-    int ih0, iw0;
-    const uint64_t *a_img;
-    {
-        const int mm = a_live ? a_m : 0;
-        const int n = mm / (p.OH * p.OW);
-        const int r = mm - n * (p.OH * p.OW);
-        const int oh = r / p.OW, ow = r - oh * p.OW;
-        ih0 = oh * p.s1 - p.p1;
-        iw0 = ow * p.s2 - p.p2;
-        a_img = p.qx + (size_t)n * p.H * p.W * p.PC * APL;
-    }
-    // B: thread fetches words (b_w0 + i*B_STEP) of filter n0 + b_row
-    const int b_row = tid % BN, b_w0 = tid / BN;
-    const bool b_live = (n0 + b_row) < p.KN;
-    const uint64_t *b_flt = p.qw + (size_t)(b_live ? n0 + b_row : 0) * p.G * BPL;
-
-    Item<APL> a_reg[A_ITEMS];
-    Item<BPL> b_reg[B_ITEMS];
-
-    auto fetch = [&](int chunk) {
-        const int g0 = chunk * p.kcw;
-#pragma unroll
-        for (int i = 0; i < A_ITEMS; i++) {
-            const int w = a_w0 + i * A_STEP;
-            const int g = g0 + w;
-            // g is uniform over the wave when BM >= 64; the tap decode is a few multiplies
-            const uint32_t tap = fastdiv((uint32_t)g, p.div_pc);
-            const int pc = g - (int)tap * p.PC;
-            const uint32_t kh = fastdiv(tap, p.div_kw);
-            const int kw = (int)tap - (int)kh * p.KW;
-            const int ih = ih0 + (int)kh, iw = iw0 + kw;
-            const bool ok = a_live && w < p.kcw && g < p.G && (unsigned)ih < (unsigned)p.H &&
-                            (unsigned)iw < (unsigned)p.W;
-            const size_t off = ok ? ((size_t)(ih * p.W + iw) * p.PC + pc) * APL : 0;
-            a_reg[i] = load_item<APL>(a_img + off, ok);
-        }
-#pragma unroll
-        for (int i = 0; i < B_ITEMS; i++) {
-            const int w = b_w0 + i * B_STEP;
-            const int g = g0 + w;
-            const bool ok = b_live && w < p.kcw && g < p.G;
-            b_reg[i] = load_item<BPL>(b_flt + (ok ? (size_t)g * BPL : 0), ok);
-        }
-    };
-    auto stage = [&](int buf) {
-        uint32_t *la = lds + buf * (A_DWORDS + B_DWORDS), *lb = la + A_DWORDS;
-#pragma unroll
-        for (int i = 0; i < A_ITEMS; i++) {
-            const int w = a_w0 + i * A_STEP;
-            if (w < kMaxChunkWords) store_item<APL, BM, kMaxQ>(la, a_reg[i], w, a_row);
-        }
-#pragma unroll
-        for (int i = 0; i < B_ITEMS; i++) {
-            const int w = b_w0 + i * B_STEP;
-            if (w < kMaxChunkWords) store_item<BPL, BN, kMaxQ>(lb, b_reg[i], w, b_row);
-        }
-    };
+    Stager st;
+    st.init(p, tid, m0, n0);
 
     // ---- accumulators --------------------------------------------------------------------
     // acc: popcount of the "negative" word (TNN/TBN/BTN) or of a^b (BNN);
@@ -274,13 +167,13 @@ __global__ __launch_bounds__(kThreads) void conv_popcount(const ConvArgs p)
             }
     };
 
-    fetch(0);
-    stage(0);
+    st.fetch(p, 0);
+    st.stage(lds);
     __syncthreads();
 
     for (int chunk = 0; chunk < p.nchunks; chunk++) {
         const bool more = chunk + 1 < p.nchunks;
-        if (more) fetch(chunk + 1);
+        if (more) st.fetch(p, chunk + 1);
 
         const uint32_t *la = lds + (chunk & 1) * (A_DWORDS + B_DWORDS), *lb = la + A_DWORDS;
         const int words_here = (p.G - chunk * p.kcw < p.kcw) ? p.G - chunk * p.kcw : p.kcw;
@@ -313,7 +206,7 @@ __global__ __launch_bounds__(kThreads) void conv_popcount(const ConvArgs p)
             }
         }
 
-        if (more) stage((chunk + 1) & 1);
+        if (more) st.stage(lds + ((chunk + 1) & 1) * (A_DWORDS + B_DWORDS));
         __syncthreads();
     }
 
@@ -442,6 +335,7 @@ void force_conv_tile(int tm, int ng)
 
 hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream)
 {
+    if (g_force_tm == 9) return launch_conv_mfma(type, args, stream);
     switch (type) {
     case 0: return launch_type<0>(args, stream);
     case 1: return launch_type<1>(args, stream);

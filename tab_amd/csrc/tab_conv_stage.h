@@ -1,0 +1,141 @@
+// Operand staging shared by the conv kernels: global memory -> registers -> LDS.
+//
+// A workgroup of 256 threads owns a BM x BN tile of Y.  K is walked in chunks of at most KCH
+// packed 64-bit words; per chunk every thread fetches a few (row, word) elements of A - the
+// im2row view of the packed activation, padding and stride in the address math, out-of-range
+// taps as all-zero words (TAB_GEMM.cuh:73-115, TAB_CPU.cpp:39,155) - and of B (the packed
+// weights), splits them into 32-bit halves and stores them k-major in LDS:
+// dword index ((plane * Q + q) * ROWS + row), q = 2 * word + half, Q = 2 * KCH.
+#pragma once
+#include "tab_common.h"
+
+namespace tab {
+
+constexpr int kConvThreads = 256;
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <int TYPE> struct Planes {
+    static constexpr int A = (TYPE == 0 || TYPE == 1) ? 2 : 1;  // activation planes (TAB_GEMM.cu:367-372)
+    static constexpr int B = (TYPE == 0 || TYPE == 2) ? 2 : 1;  // weight planes (TAB_GEMM.cu:374-379)
+};
+
+// One packed word (all planes) of one row of an operand, held in registers between the
+// global load and the LDS store.  Memory order is [plane][half] as 64-bit words.
+template <int PL> struct Item {
+    uint32_t d[2 * PL];
+};
+
+template <int PL>
+__device__ __forceinline__ Item<PL> load_item(const uint64_t *p, bool valid)
+{
+    Item<PL> it;
+    if (PL == 2) {
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (valid) v = *reinterpret_cast<const u32x4 *>(p);
+        it.d[0] = v[0]; it.d[1] = v[1]; it.d[2] = v[2]; it.d[3] = v[3];
+    } else {
+        u32x2 v = {0u, 0u};
+        if (valid) v = *reinterpret_cast<const u32x2 *>(p);
+        it.d[0] = v[0]; it.d[1] = v[1];
+    }
+    return it;
+}
+
+template <int PL, int ROWS, int Q>
+__device__ __forceinline__ void store_item(uint32_t *lds, const Item<PL> &it, int word, int row)
+{
+#pragma unroll
+    for (int pl = 0; pl < PL; pl++)
+#pragma unroll
+        for (int half = 0; half < 2; half++)
+            lds[((pl * Q) + 2 * word + half) * ROWS + row] = it.d[pl * 2 + half];
+}
+
+template <int TYPE, int BM, int BN, int KCH>
+struct TileStager {
+    static constexpr int APL = Planes<TYPE>::A, BPL = Planes<TYPE>::B;
+    static constexpr int Q = 2 * KCH;  // 32-bit k-slices per chunk
+    static constexpr int A_DWORDS = APL * Q * BM, B_DWORDS = BPL * Q * BN;
+    static constexpr int A_STEP = kConvThreads / BM, B_STEP = kConvThreads / BN;  // words per pass over the rows
+    static constexpr int A_ITEMS = (KCH + A_STEP - 1) / A_STEP, B_ITEMS = (KCH + B_STEP - 1) / B_STEP;
+    static_assert(kConvThreads % BM == 0 && kConvThreads % BN == 0, "tile rows must divide the workgroup");
+
+    // A: this thread fetches words (a_w0 + i*A_STEP) of output pixel m0 + a_row
+    int a_row, a_w0, ih0, iw0;
+    bool a_live;
+    const uint64_t *a_img;
+    // B: this thread fetches words (b_w0 + i*B_STEP) of filter n0 + b_row
+    int b_row, b_w0;
+    bool b_live;
+    const uint64_t *b_flt;
+    Item<APL> a_reg[A_ITEMS];
+    Item<BPL> b_reg[B_ITEMS];
+
+    __device__ __forceinline__ void init(const ConvArgs &p, int tid, int m0, int n0)
+    {
+        a_row = tid % BM;
+        a_w0 = tid / BM;
+        const int a_m = m0 + a_row;
+        a_live = a_m < p.M;
+        const int mm = a_live ? a_m : 0;
+        const int n = mm / (p.OH * p.OW);
+        const int r = mm - n * (p.OH * p.OW);
+        const int oh = r / p.OW, ow = r - oh * p.OW;
+        ih0 = oh * p.s1 - p.p1;
+        iw0 = ow * p.s2 - p.p2;
+        a_img = p.qx + (size_t)n * p.H * p.W * p.PC * APL;
+        b_row = tid % BN;
+        b_w0 = tid / BN;
+        b_live = (n0 + b_row) < p.KN;
+        b_flt = p.qw + (size_t)(b_live ? n0 + b_row : 0) * p.G * BPL;
+    }
+
+    // issue the global loads of one chunk into registers
+    __device__ __forceinline__ void fetch(const ConvArgs &p, int chunk)
+    {
+        const int g0 = chunk * p.kcw;
+#pragma unroll
+        for (int i = 0; i < A_ITEMS; i++) {
+            const int w = a_w0 + i * A_STEP;
+            const int g = g0 + w;
+            // g is uniform over the wave when BM >= 64; the tap decode is a few multiplies
+            const uint32_t tap = fastdiv((uint32_t)g, p.div_pc);
+            const int pc = g - (int)tap * p.PC;
+            const uint32_t kh = fastdiv(tap, p.div_kw);
+            const int kw = (int)tap - (int)kh * p.KW;
+            const int ih = ih0 + (int)kh, iw = iw0 + kw;
+            const bool ok = a_live && w < p.kcw && g < p.G && (unsigned)ih < (unsigned)p.H &&
+                            (unsigned)iw < (unsigned)p.W;
+            const size_t off = ok ? ((size_t)(ih * p.W + iw) * p.PC + pc) * APL : 0;
+            a_reg[i] = load_item<APL>(a_img + off, ok);
+        }
+#pragma unroll
+        for (int i = 0; i < B_ITEMS; i++) {
+            const int w = b_w0 + i * B_STEP;
+            const int g = g0 + w;
+            const bool ok = b_live && w < p.kcw && g < p.G;
+            b_reg[i] = load_item<BPL>(b_flt + (ok ? (size_t)g * BPL : 0), ok);
+        }
+    }
+
+    // write the fetched chunk to an LDS buffer of A_DWORDS + B_DWORDS dwords
+    __device__ __forceinline__ void stage(uint32_t *buf) const
+    {
+        uint32_t *la = buf, *lb = buf + A_DWORDS;
+#pragma unroll
+        for (int i = 0; i < A_ITEMS; i++) {
+            const int w = a_w0 + i * A_STEP;
+            if (w < KCH) store_item<APL, BM, Q>(la, a_reg[i], w, a_row);
+        }
+#pragma unroll
+        for (int i = 0; i < B_ITEMS; i++) {
+            const int w = b_w0 + i * B_STEP;
+            if (w < KCH) store_item<BPL, BN, Q>(lb, b_reg[i], w, b_row);
+        }
+    }
+};
+
+}  // namespace tab
