@@ -49,7 +49,10 @@ struct ConvArgs {
 // Launchers (tab_conv.hip / tab_quantize.hip); they enqueue on `stream` and return the
 // launch status.
 hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream);
-hipError_t launch_conv_mfma(int type, const ConvArgs &args, hipStream_t stream);  // matrix-core variant, 128x128 tiles
+// Matrix-core (FP4 MFMA) variant; shape picks the workgroup tile.  conv_mfma_exact() says whether K is
+// short enough for its fp32 accumulators to hold every partial sum exactly.
+bool conv_mfma_exact(const ConvArgs &args);
+hipError_t launch_conv_mfma(int type, const ConvArgs &args, int shape, hipStream_t stream);
 hipError_t launch_quantize(const float *x, const float *ths, int bitwidth, long pixels_per_item,
                            long items, int C, uint64_t *qx, int32_t *btn, hipStream_t stream);
 

@@ -335,7 +335,7 @@ void force_conv_tile(int tm, int ng)
 
 hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream)
 {
-    if (g_force_tm == 9) return launch_conv_mfma(type, args, stream);
+    if (g_force_tm == 9) return launch_conv_mfma(type, args, g_force_ng, stream);
     switch (type) {
     case 0: return launch_type<0>(args, stream);
     case 1: return launch_type<1>(args, stream);

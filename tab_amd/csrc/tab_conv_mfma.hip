@@ -1,202 +1,204 @@
 // Matrix-core variant of the fused pad + im2row + bitwise GEMM: the packed bit planes are
-// expanded to int8 in registers and multiplied with v_mfma_i32_32x32x32_i8.
+// expanded in registers to FP4 (E2M1) operands of v_mfma_f32_32x32x64_f8f6f4.
 //
-// The four TAB formulas (TAB_GEMM.cu:25-147) written as integer dot products, with
-// a_k = a1*(1 - 2*a0), b_k = b1*(1 - 2*b0) the decoded ternary values (any bit pattern) and
-// a01, b01 the raw bits of a binary operand:
-//   TNN  y = sum a_k*b_k
-//   TBN  y = sum a_k - 2 * sum a_k*b01
-//   BTN  y = btn[n] - 2 * (sum a01*b_k + popcount(b0 & b1))
-//   BNN  y = NUM - 2 * (popcount(a) + popcount(b) - 2 * sum a01*b01)
-// All sums are exact in int32.  Zero-padded taps and the unused high bits of a tail word are
-// zero bits on both sides and contribute nothing, as in the popcount formulas.
+// With a_k = a1*(1 - 2*a0) the decoded ternary value (any bit pattern of the two planes) and
+// (1 - 2*a) the value of a binary bit, the four TAB formulas (TAB_GEMM.cu:25-147) are plain
+// dot products D over all 64*G packed bit positions:
+//   TNN  sum popc(a1&b1) - 2*sum popc((a0^b0)&a1&b1)  = D
+//   TBN  sum popc(a1)    - 2*sum popc((a0^b)&a1)      = D
+//   BTN  btn[n]          - 2*sum popc((a^b0)&b1)      = D + btn[n] - popc(b1 of filter n)
+//   BNN  NUM             - 2*sum popc(a^b)            = D - (64*G - NUM)
+// Zero words (padded taps, rows past M) decode to 0 for a ternary and to +1 for a binary
+// operand, which is what the reference's padding means (TAB_CPU.cpp:39,155).
 //
-// Tiling: 256 threads, 128x128 tile of Y, operands staged in LDS exactly as for the popcount
-// kernel (tab_conv_stage.h).  Wave w owns the 64x64 quadrant (w&1, w>>1) as 2x2 MFMA tiles.
-// Per 32-bit k-slice a lane reads the slice word of its row (A) / column (B) - lane%32 - and
-// expands the 16 bits lane/32 selects into the 16 int8 of its MFMA operand: 4 bits -> 4 bytes
-// with one v_bfe, one 24-bit multiply by 0x204081 (copies of the nibble at bit 0, 7, 14, 21)
-// and one mask.
+// E2M1 nibble = sign, 2 exponent bits, 1 mantissa bit: 0001 = 0.5, 0010 = 1, 0100 = 2, and a
+// lone sign bit is -0.  Bit j of every nibble of a 32-bit slice goes to operand dword j with
+// one AND (plus a shift where the bit has to move): magnitude weights (0.5, 1, 2, 2) on the A
+// side meet (2, 1, 0.5, 0.5) on the B side, so every product is exactly +-1 or 0.  The order
+// of k inside an operand is irrelevant as long as A and B agree, and they do: both come from
+// the same bit of the same slice.  All partial sums are integers below 2^24 in magnitude
+// (64*G is bounded by the launcher), hence exact in the fp32 accumulators.
+//
+// Tiling: 256 threads = WM x WN waves, each wave TM x TN MFMA tiles of 32x32; operands are
+// staged in LDS exactly as for the popcount kernel (tab_conv_stage.h).  Per 64-bit word a lane
+// reads the 32-bit half lane/32 selects of its row (A) or column (B), lane%32.
 #include "tab_conv_stage.h"
 
 namespace tab {
 namespace {
 
-typedef int i32x4 __attribute__((ext_vector_type(4)));
-typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-// bits [shift, shift+16) of word -> 16 bytes of 0/1
-__device__ __forceinline__ i32x4 expand01(uint32_t word, uint32_t shift)
+constexpr uint32_t kBit0 = 0x11111111u, kBit1 = 0x22222222u, kBit2 = 0x44444444u, kBit3 = 0x88888888u;
+
+// SIDE 0 = activation (weights 0.5, 1, 2, 2), SIDE 1 = weight operand (2, 1, 0.5, 0.5)
+template <int SIDE>
+__device__ __forceinline__ i32x8 expand_binary(uint32_t w)
 {
-    i32x4 r;
-#pragma unroll
-    for (int d = 0; d < 4; d++) {
-        const uint32_t nib = __builtin_amdgcn_ubfe(word, shift + 4 * d, 4);
-        r[d] = (int)(__umul24(nib, 0x00204081u) & 0x01010101u);
+    constexpr uint32_t m0 = SIDE ? kBit2 : kBit0, m2 = SIDE ? kBit0 : kBit2;
+    i32x8 r = {0, 0, 0, 0, 0, 0, 0, 0};
+    r[0] = (int)(((w << 3) & kBit3) | m0);
+    r[1] = (int)(((w << 2) & kBit3) | kBit1);
+    r[2] = (int)(((w << 1) & kBit3) | m2);
+    r[3] = (int)((w & kBit3) | m2);
+    return r;
+}
+
+template <int SIDE>
+__device__ __forceinline__ i32x8 expand_ternary(uint32_t s, uint32_t z)
+{
+    i32x8 r = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (SIDE == 0) {
+        r[0] = (int)((z & kBit0) | ((s << 3) & kBit3));
+        r[1] = (int)((z & kBit1) | ((s << 2) & kBit3));
+        r[2] = (int)((z & kBit2) | ((s << 1) & kBit3));
+        r[3] = (int)(((z >> 1) & kBit2) | (s & kBit3));
+    } else {
+        r[0] = (int)(((z << 2) & kBit2) | ((s << 3) & kBit3));
+        r[1] = (int)((z & kBit1) | ((s << 2) & kBit3));
+        r[2] = (int)(((z >> 2) & kBit0) | ((s << 1) & kBit3));
+        r[3] = (int)(((z >> 3) & kBit0) | (s & kBit3));
     }
     return r;
 }
 
-// the same 16 positions of a ternary operand -> bytes +1, 0, -1 (0xFF)
-__device__ __forceinline__ i32x4 expand_ternary(uint32_t sign, uint32_t nz, uint32_t shift)
-{
-    const i32x4 z = expand01(nz, shift), g = expand01(sign & nz, shift);
-    i32x4 r;
-#pragma unroll
-    for (int d = 0; d < 4; d++) r[d] = z[d] | ((g[d] << 8) - g[d]);  // (x << 8) - x = 0xFF per set byte
-    return r;
-}
-
-__device__ __forceinline__ int popcount16(uint32_t word, uint32_t shift)
-{
-    return __builtin_popcount(__builtin_amdgcn_ubfe(word, shift, 16));
-}
-
-template <int TYPE, int KCH>
+template <int TYPE, int WM, int WN, int TM, int TN, int KCH>
 __global__ __launch_bounds__(kConvThreads) void conv_mfma(const ConvArgs p)
 {
+    static_assert(WM * WN * 64 == kConvThreads, "four waves");
     constexpr int APL = Planes<TYPE>::A, BPL = Planes<TYPE>::B;
-    constexpr int BM = 128, BN = 128;
+    constexpr int BM = 32 * WM * TM, BN = 32 * WN * TN;
     using Stager = TileStager<TYPE, BM, BN, KCH>;
     constexpr int Q = Stager::Q, A_DWORDS = Stager::A_DWORDS, B_DWORDS = Stager::B_DWORDS;
 
     __shared__ __attribute__((aligned(16))) uint32_t lds[2 * (A_DWORDS + B_DWORDS)];
-    __shared__ int row_side[4][64];  // per wave: row-side sums for the epilogue
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
-    const int r = lane & 31;                  // row of an A tile / column of a B tile
-    const uint32_t shift = 16 * (lane >> 5);  // which 16 of the 32 k this lane feeds
-    const int wm = wave & 1, wn = wave >> 1;
+    const int r = lane & 31;   // row of an A tile / column of a B tile
+    const int kb = lane >> 5;  // which 32-bit half of the word this lane feeds
+    const int wm = wave % WM, wn = wave / WM;
     const int tile_m = blockIdx.x % p.tiles_m, tile_n = blockIdx.x / p.tiles_m;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
     Stager st;
     st.init(p, tid, m0, n0);
 
-    i32x16 acc[2][2];
+    f32x16 acc[TM][TN];
 #pragma unroll
-    for (int mt = 0; mt < 2; mt++)
+    for (int mt = 0; mt < TM; mt++)
 #pragma unroll
-        for (int nt = 0; nt < 2; nt++)
+        for (int nt = 0; nt < TN; nt++)
 #pragma unroll
-            for (int e = 0; e < 16; e++) acc[mt][nt][e] = 0;
-    int a_side[2] = {0, 0}, b_side[2] = {0, 0};
+            for (int e = 0; e < 16; e++) acc[mt][nt][e] = 0.f;
+    int b_nonzero[TN];  // BTN: bits set in the nonzero plane of this lane's half of its filters
+#pragma unroll
+    for (int nt = 0; nt < TN; nt++) b_nonzero[nt] = 0;
 
     st.fetch(p, 0);
     st.stage(lds);
     __syncthreads();
 
+    const int a_off = wm * (32 * TM) + r, b_off = wn * (32 * TN) + r;
     for (int chunk = 0; chunk < p.nchunks; chunk++) {
         const bool more = chunk + 1 < p.nchunks;
         if (more) st.fetch(p, chunk + 1);
 
         const uint32_t *la = lds + (chunk & 1) * (A_DWORDS + B_DWORDS), *lb = la + A_DWORDS;
         const int words_here = (p.G - chunk * p.kcw < p.kcw) ? p.G - chunk * p.kcw : p.kcw;
-        const int nq = 2 * words_here;
-        for (int q = 0; q < nq; q++) {
-            uint32_t aw[APL][2], bw[BPL][2];
+        for (int w = 0; w < words_here; w++) {
+            const int q = 2 * w + kb;
+            i32x8 af[TM], bf[TN];
 #pragma unroll
-            for (int pl = 0; pl < APL; pl++)
+            for (int mt = 0; mt < TM; mt++) {
+                const uint32_t a0 = la[q * BM + a_off + mt * 32];
+                if (APL == 2) af[mt] = expand_ternary<0>(a0, la[(Q + q) * BM + a_off + mt * 32]);
+                else af[mt] = expand_binary<0>(a0);
+            }
 #pragma unroll
-                for (int mt = 0; mt < 2; mt++) aw[pl][mt] = la[(pl * Q + q) * BM + wm * 64 + mt * 32 + r];
-#pragma unroll
-            for (int pl = 0; pl < BPL; pl++)
-#pragma unroll
-                for (int nt = 0; nt < 2; nt++) bw[pl][nt] = lb[(pl * Q + q) * BN + wn * 64 + nt * 32 + r];
-
-            i32x4 af[2], bf[2];
-#pragma unroll
-            for (int t = 0; t < 2; t++) {
-                if (APL == 2) {
-                    af[t] = expand_ternary(aw[0][t], aw[APL - 1][t], shift);
-                    if (TYPE == 1)  // sum of a_k over this lane's 16 positions
-                        a_side[t] += popcount16(aw[APL - 1][t], shift) - 2 * popcount16(aw[0][t] & aw[APL - 1][t], shift);
-                } else {
-                    af[t] = expand01(aw[0][t], shift);
-                    if (TYPE == 3) a_side[t] += popcount16(aw[0][t], shift);
-                }
+            for (int nt = 0; nt < TN; nt++) {
+                const uint32_t b0 = lb[q * BN + b_off + nt * 32];
                 if (BPL == 2) {
-                    bf[t] = expand_ternary(bw[0][t], bw[BPL - 1][t], shift);
-                    if (TYPE == 2) b_side[t] += popcount16(bw[0][t] & bw[BPL - 1][t], shift);
+                    const uint32_t b1 = lb[(Q + q) * BN + b_off + nt * 32];
+                    bf[nt] = expand_ternary<1>(b0, b1);
+                    if (TYPE == 2) b_nonzero[nt] += __builtin_popcount(b1);
                 } else {
-                    bf[t] = expand01(bw[0][t], shift);
-                    if (TYPE == 3) b_side[t] += popcount16(bw[0][t], shift);
+                    bf[nt] = expand_binary<1>(b0);
                 }
             }
 #pragma unroll
-            for (int mt = 0; mt < 2; mt++)
+            for (int mt = 0; mt < TM; mt++)
 #pragma unroll
-                for (int nt = 0; nt < 2; nt++)
-                    acc[mt][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[mt], bf[nt], acc[mt][nt], 0, 0, 0);
+                for (int nt = 0; nt < TN; nt++)
+                    acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[mt], bf[nt], acc[mt][nt], 4, 4, 0, 0, 0, 0);
         }
 
         if (more) st.stage(lds + ((chunk + 1) & 1) * (A_DWORDS + B_DWORDS));
         __syncthreads();
     }
 
-    // ---- epilogue ------------------------------------------------------------------------
-    // the two lanes r and r+32 hold the two halves of every side sum
+    // ---- epilogue: accumulator element 4*j + i of lane (kb, r) is C[8*j + 4*kb + i][r] -------
 #pragma unroll
-    for (int t = 0; t < 2; t++) {
-        a_side[t] += __shfl_xor(a_side[t], 32, 64);
-        b_side[t] += __shfl_xor(b_side[t], 32, 64);
-    }
-    if (TYPE == 1 || TYPE == 3) {  // row sums live in the lane of their row; outputs need them by row index
-        if (lane < 32) {
-            row_side[wave][r] = a_side[0];
-            row_side[wave][32 + r] = a_side[1];
-        }
-        __syncthreads();
-    }
-    // accumulator element 4*j + i of lane (kb, r) is C[8*j + 4*kb + i][r]
-#pragma unroll
-    for (int nt = 0; nt < 2; nt++) {
-        const int col = n0 + wn * 64 + nt * 32 + r;
+    for (int nt = 0; nt < TN; nt++) {
+        const int col = n0 + wn * (32 * TN) + nt * 32 + r;
         const bool col_ok = col < p.KN;
-        const int bias = (TYPE == 2 && col_ok) ? p.btn[col] : 0;
+        float bias = 0.f;
+        if (TYPE == 2) {
+            const int nonzero = b_nonzero[nt] + __shfl_xor(b_nonzero[nt], 32, 64);
+            bias = (float)((col_ok ? p.btn[col] : 0) - nonzero);
+        }
+        if (TYPE == 3) bias = (float)(p.num - 64 * p.G);
 #pragma unroll
-        for (int mt = 0; mt < 2; mt++)
+        for (int mt = 0; mt < TM; mt++)
 #pragma unroll
             for (int j = 0; j < 4; j++)
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    const int row_l = mt * 32 + 8 * j + 4 * (lane >> 5) + i;
-                    const int m = m0 + wm * 64 + row_l;
-                    const int d = acc[mt][nt][4 * j + i];
-                    int v;
-                    if (TYPE == 0) v = d;
-                    else if (TYPE == 1) v = row_side[wave][row_l] - 2 * d;
-                    else if (TYPE == 2) v = bias - 2 * (d + b_side[nt]);
-                    else v = p.num - 2 * (row_side[wave][row_l] + b_side[nt] - 2 * d);
-                    if (col_ok && m < p.M) p.y[(size_t)m * p.KN + col] = (float)v;
+                    const int m = m0 + wm * (32 * TM) + mt * 32 + 8 * j + 4 * kb + i;
+                    if (col_ok && m < p.M) p.y[(size_t)m * p.KN + col] = acc[mt][nt][4 * j + i] + bias;
                 }
     }
 }
 
-template <int TYPE>
-hipError_t launch_mfma(ConvArgs a, hipStream_t stream)
+template <int TYPE, int WM, int WN, int TM, int TN, int KCH>
+hipError_t launch_mfma_tile(ConvArgs a, hipStream_t stream)
 {
-    constexpr int KCH = 4;
+    constexpr int BM = 32 * WM * TM, BN = 32 * WN * TN;
     a.nchunks = (a.G + KCH - 1) / KCH;
     a.kcw = (a.G + a.nchunks - 1) / a.nchunks;
     a.nchunks = (a.G + a.kcw - 1) / a.kcw;
-    a.tiles_m = (a.M + 127) / 128;
-    const long blocks = (long)a.tiles_m * ((a.KN + 127) / 128);
+    a.tiles_m = (a.M + BM - 1) / BM;
+    const long blocks = (long)a.tiles_m * ((a.KN + BN - 1) / BN);
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
-    conv_mfma<TYPE, KCH><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
+    conv_mfma<TYPE, WM, WN, TM, TN, KCH><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
     return hipGetLastError();
+}
+
+template <int TYPE>
+hipError_t launch_mfma(const ConvArgs &a, int shape, hipStream_t stream)
+{
+    switch (shape) {
+    case 0: return launch_mfma_tile<TYPE, 2, 2, 2, 2, 4>(a, stream);  // 128 x 128
+    case 1: return launch_mfma_tile<TYPE, 4, 1, 1, 2, 4>(a, stream);  // 128 x 64
+    case 2: return launch_mfma_tile<TYPE, 2, 2, 1, 1, 4>(a, stream);  //  64 x 64
+    case 3: return launch_mfma_tile<TYPE, 2, 2, 1, 2, 4>(a, stream);  //  64 x 128
+    default: return hipErrorInvalidValue;
+    }
 }
 
 }  // namespace
 
-hipError_t launch_conv_mfma(int type, const ConvArgs &args, hipStream_t stream)
+bool conv_mfma_exact(const ConvArgs &a) { return (long)a.G * 64 <= (1L << 22); }
+
+hipError_t launch_conv_mfma(int type, const ConvArgs &args, int shape, hipStream_t stream)
 {
+    if (!conv_mfma_exact(args)) return hipErrorInvalidValue;
     switch (type) {
-    case 0: return launch_mfma<0>(args, stream);
-    case 1: return launch_mfma<1>(args, stream);
-    case 2: return launch_mfma<2>(args, stream);
-    case 3: return launch_mfma<3>(args, stream);
+    case 0: return launch_mfma<0>(args, shape, stream);
+    case 1: return launch_mfma<1>(args, shape, stream);
+    case 2: return launch_mfma<2>(args, shape, stream);
+    case 3: return launch_mfma<3>(args, shape, stream);
     default: return hipErrorInvalidValue;
     }
 }
