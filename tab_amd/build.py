@@ -6,7 +6,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libtab_amd.so")
-SOURCES = ["tab_capi.hip", "tab_conv.hip", "tab_conv_mfma.hip", "tab_quantize.hip"]
+SOURCES = ["tab_capi.hip", "tab_conv.hip", "tab_conv_mfma_tnn.hip", "tab_conv_mfma_tbn.hip", "tab_conv_mfma_btn.hip",
+           "tab_conv_mfma_bnn.hip", "tab_quantize.hip"]
+OBJ_DIR = os.path.join(LIB_DIR, "obj")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -packed-fp32-ops: keep the compiler from forming packed-FP32 VALU ops from float code.
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall",
@@ -58,16 +60,27 @@ def build_torch_extension(verbose=False):
     return extension_path()
 
 
-def build_library(verbose=False):
-    """Compile every HIP source and link libtab_amd.so. Always recompiles."""
-    os.makedirs(LIB_DIR, exist_ok=True)
-    cmd = [HIPCC] + HIP_FLAGS + ["-shared", "-o", LIB_PATH] + [os.path.join(CSRC, s) for s in SOURCES]
+def _hipcc(cmd):
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l)
     if proc.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + out)
-    if verbose and out.strip():
-        print(out)
+        raise RuntimeError("hipcc failed: " + " ".join(cmd) + "\n" + out)
+    return out
+
+
+def build_library(verbose=False):
+    """Compile every HIP source (one hipcc per source, side by side) and link libtab_amd.so.
+    Always recompiles."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    objs = [os.path.join(OBJ_DIR, s.replace(".hip", ".o")) for s in SOURCES]
+    cmds = [[HIPCC] + HIP_FLAGS + ["-c", os.path.join(CSRC, s), "-o", o] for s, o in zip(SOURCES, objs)]
+    with ThreadPoolExecutor(max_workers=min(8, len(cmds))) as pool:
+        outs = list(pool.map(_hipcc, cmds))
+    outs.append(_hipcc([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs))
+    if verbose and any(o.strip() for o in outs):
+        print("\n".join(o for o in outs if o.strip()))
     return LIB_PATH
 
 

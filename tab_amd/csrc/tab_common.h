@@ -53,6 +53,10 @@ hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream);
 // short enough for its fp32 accumulators to hold every partial sum exactly.
 bool conv_mfma_exact(const ConvArgs &args);
 hipError_t launch_conv_mfma(int type, const ConvArgs &args, int shape, hipStream_t stream);
+hipError_t launch_conv_mfma_tnn(const ConvArgs &args, int shape, hipStream_t stream);
+hipError_t launch_conv_mfma_tbn(const ConvArgs &args, int shape, hipStream_t stream);
+hipError_t launch_conv_mfma_btn(const ConvArgs &args, int shape, hipStream_t stream);
+hipError_t launch_conv_mfma_bnn(const ConvArgs &args, int shape, hipStream_t stream);
 hipError_t launch_quantize(const float *x, const float *ths, int bitwidth, long pixels_per_item,
                            long items, int C, uint64_t *qx, int32_t *btn, hipStream_t stream);
 

@@ -333,6 +333,20 @@ void force_conv_tile(int tm, int ng)
     g_force_ng = ng;
 }
 
+bool conv_mfma_exact(const ConvArgs &a) { return (long)a.G * 64 <= (1L << 22); }
+
+hipError_t launch_conv_mfma(int type, const ConvArgs &args, int shape, hipStream_t stream)
+{
+    if (!conv_mfma_exact(args)) return hipErrorInvalidValue;
+    switch (type) {
+    case 0: return launch_conv_mfma_tnn(args, shape, stream);
+    case 1: return launch_conv_mfma_tbn(args, shape, stream);
+    case 2: return launch_conv_mfma_btn(args, shape, stream);
+    case 3: return launch_conv_mfma_bnn(args, shape, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
 hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream)
 {
     if (g_force_tm == 9) return launch_conv_mfma(type, args, g_force_ng, stream);

@@ -22,6 +22,7 @@
 // Tiling: 256 threads = WM x WN waves, each wave TM x TN MFMA tiles of 32x32; operands are
 // staged in LDS exactly as for the popcount kernel (tab_conv_stage.h).  Per 64-bit word a lane
 // reads the 32-bit half lane/32 selects of its row (A) or column (B), lane%32.
+#pragma once
 #include "tab_conv_stage.h"
 
 namespace tab {
@@ -32,16 +33,26 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr uint32_t kBit0 = 0x11111111u, kBit1 = 0x22222222u, kBit2 = 0x44444444u, kBit3 = 0x88888888u;
 
+// (a & m) | c in one instruction.  This ISA takes no literal in a three-operand VALU instruction and
+// only one scalar register, so the mask rides in an SGPR and the other two operands in VGPRs; left
+// to itself the compiler emits a separate v_and and v_or with two literals.
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t m, uint32_t c)
+{
+    uint32_t r;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(m), "v"(c));
+    return r;
+}
+
 // SIDE 0 = activation (weights 0.5, 1, 2, 2), SIDE 1 = weight operand (2, 1, 0.5, 0.5)
 template <int SIDE>
 __device__ __forceinline__ i32x8 expand_binary(uint32_t w)
 {
     constexpr uint32_t m0 = SIDE ? kBit2 : kBit0, m2 = SIDE ? kBit0 : kBit2;
     i32x8 r = {0, 0, 0, 0, 0, 0, 0, 0};
-    r[0] = (int)(((w << 3) & kBit3) | m0);
-    r[1] = (int)(((w << 2) & kBit3) | kBit1);
-    r[2] = (int)(((w << 1) & kBit3) | m2);
-    r[3] = (int)((w & kBit3) | m2);
+    r[0] = (int)and_or(w << 3, kBit3, m0);
+    r[1] = (int)and_or(w << 2, kBit3, kBit1);
+    r[2] = (int)and_or(w << 1, kBit3, m2);
+    r[3] = (int)and_or(w, kBit3, m2);
     return r;
 }
 
@@ -50,15 +61,15 @@ __device__ __forceinline__ i32x8 expand_ternary(uint32_t s, uint32_t z)
 {
     i32x8 r = {0, 0, 0, 0, 0, 0, 0, 0};
     if (SIDE == 0) {
-        r[0] = (int)((z & kBit0) | ((s << 3) & kBit3));
-        r[1] = (int)((z & kBit1) | ((s << 2) & kBit3));
-        r[2] = (int)((z & kBit2) | ((s << 1) & kBit3));
-        r[3] = (int)(((z >> 1) & kBit2) | (s & kBit3));
+        r[0] = (int)and_or(s << 3, kBit3, z & kBit0);
+        r[1] = (int)and_or(s << 2, kBit3, z & kBit1);
+        r[2] = (int)and_or(s << 1, kBit3, z & kBit2);
+        r[3] = (int)and_or(s, kBit3, (z >> 1) & kBit2);
     } else {
-        r[0] = (int)(((z << 2) & kBit2) | ((s << 3) & kBit3));
-        r[1] = (int)((z & kBit1) | ((s << 2) & kBit3));
-        r[2] = (int)(((z >> 2) & kBit0) | ((s << 1) & kBit3));
-        r[3] = (int)(((z >> 3) & kBit0) | (s & kBit3));
+        r[0] = (int)and_or(s << 3, kBit3, (z << 2) & kBit2);
+        r[1] = (int)and_or(s << 2, kBit3, z & kBit1);
+        r[2] = (int)and_or(s << 1, kBit3, (z >> 2) & kBit0);
+        r[3] = (int)and_or(s, kBit3, (z >> 3) & kBit0);
     }
     return r;
 }
@@ -105,27 +116,34 @@ __global__ __launch_bounds__(kConvThreads) void conv_mfma(const ConvArgs p)
         const bool more = chunk + 1 < p.nchunks;
         if (more) st.fetch(p, chunk + 1);
 
-        const uint32_t *la = lds + (chunk & 1) * (A_DWORDS + B_DWORDS), *lb = la + A_DWORDS;
-        const int words_here = (p.G - chunk * p.kcw < p.kcw) ? p.G - chunk * p.kcw : p.kcw;
-        for (int w = 0; w < words_here; w++) {
+        // Every chunk is exactly KCH words: the stager zero-fills words past the end of K, which add
+        // nothing for a ternary operand and +64 per word for binary x binary (the BNN bias below
+        // counts them).  LDS reads run one word ahead of the matrix cores.
+        const uint32_t *la = lds + (chunk & 1) * (A_DWORDS + B_DWORDS) + a_off, *lb = la - a_off + A_DWORDS + b_off;
+        uint32_t a_w[KCH][APL][TM], b_w[KCH][BPL][TN];
+        auto read_word = [&](int w) {
             const int q = 2 * w + kb;
+#pragma unroll
+            for (int pl = 0; pl < APL; pl++)
+#pragma unroll
+                for (int mt = 0; mt < TM; mt++) a_w[w][pl][mt] = la[(pl * Q + q) * BM + mt * 32];
+#pragma unroll
+            for (int pl = 0; pl < BPL; pl++)
+#pragma unroll
+                for (int nt = 0; nt < TN; nt++) b_w[w][pl][nt] = lb[(pl * Q + q) * BN + nt * 32];
+        };
+        read_word(0);
+#pragma unroll
+        for (int w = 0; w < KCH; w++) {
+            if (w + 1 < KCH) read_word(w + 1);
             i32x8 af[TM], bf[TN];
 #pragma unroll
-            for (int mt = 0; mt < TM; mt++) {
-                const uint32_t a0 = la[q * BM + a_off + mt * 32];
-                if (APL == 2) af[mt] = expand_ternary<0>(a0, la[(Q + q) * BM + a_off + mt * 32]);
-                else af[mt] = expand_binary<0>(a0);
-            }
+            for (int mt = 0; mt < TM; mt++)
+                af[mt] = (APL == 2) ? expand_ternary<0>(a_w[w][0][mt], a_w[w][APL - 1][mt]) : expand_binary<0>(a_w[w][0][mt]);
 #pragma unroll
             for (int nt = 0; nt < TN; nt++) {
-                const uint32_t b0 = lb[q * BN + b_off + nt * 32];
-                if (BPL == 2) {
-                    const uint32_t b1 = lb[(Q + q) * BN + b_off + nt * 32];
-                    bf[nt] = expand_ternary<1>(b0, b1);
-                    if (TYPE == 2) b_nonzero[nt] += __builtin_popcount(b1);
-                } else {
-                    bf[nt] = expand_binary<1>(b0);
-                }
+                bf[nt] = (BPL == 2) ? expand_ternary<1>(b_w[w][0][nt], b_w[w][BPL - 1][nt]) : expand_binary<1>(b_w[w][0][nt]);
+                if (TYPE == 2) b_nonzero[nt] += __builtin_popcount(b_w[w][BPL - 1][nt]);
             }
 #pragma unroll
             for (int mt = 0; mt < TM; mt++)
@@ -139,35 +157,51 @@ __global__ __launch_bounds__(kConvThreads) void conv_mfma(const ConvArgs p)
     }
 
     // ---- epilogue: accumulator element 4*j + i of lane (kb, r) is C[8*j + 4*kb + i][r] -------
+    const int wave_m0 = m0 + wm * (32 * TM), wave_n0 = n0 + wn * (32 * TN);
+    const bool whole = wave_m0 + 32 * TM <= p.M && wave_n0 + 32 * TN <= p.KN;  // wave-uniform
 #pragma unroll
     for (int nt = 0; nt < TN; nt++) {
-        const int col = n0 + wn * (32 * TN) + nt * 32 + r;
+        const int col = wave_n0 + nt * 32 + r;
         const bool col_ok = col < p.KN;
         float bias = 0.f;
         if (TYPE == 2) {
             const int nonzero = b_nonzero[nt] + __shfl_xor(b_nonzero[nt], 32, 64);
             bias = (float)((col_ok ? p.btn[col] : 0) - nonzero);
         }
-        if (TYPE == 3) bias = (float)(p.num - 64 * p.G);
+        if (TYPE == 3) bias = (float)(p.num - 64 * p.nchunks * KCH);
+        float *out = p.y + (size_t)(wave_m0 + 4 * kb) * p.KN + col;
 #pragma unroll
         for (int mt = 0; mt < TM; mt++)
 #pragma unroll
             for (int j = 0; j < 4; j++)
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    const int m = m0 + wm * (32 * TM) + mt * 32 + 8 * j + 4 * kb + i;
-                    if (col_ok && m < p.M) p.y[(size_t)m * p.KN + col] = acc[mt][nt][4 * j + i] + bias;
+                    const int row = mt * 32 + 8 * j + i;  // + 4*kb, already in `out`
+                    const float v = acc[mt][nt][4 * j + i] + bias;
+                    if (whole) out[(size_t)row * p.KN] = v;
+                    else if (col_ok && wave_m0 + 4 * kb + row < p.M) out[(size_t)row * p.KN] = v;
                 }
     }
+}
+
+// Chunk length for G words: 1..4, the one with the least padded work (a barrier is priced as half a
+// word), longer chunks on ties.
+inline int mfma_chunk_words(int G)
+{
+    int best = 4, best_cost = 0x7fffffff;
+    for (int k = 4; k >= 1; k--) {
+        const int cost = ((G + k - 1) / k) * (2 * k + 1);
+        if (cost < best_cost) { best = k; best_cost = cost; }
+    }
+    return best;
 }
 
 template <int TYPE, int WM, int WN, int TM, int TN, int KCH>
 hipError_t launch_mfma_tile(ConvArgs a, hipStream_t stream)
 {
     constexpr int BM = 32 * WM * TM, BN = 32 * WN * TN;
+    a.kcw = KCH;
     a.nchunks = (a.G + KCH - 1) / KCH;
-    a.kcw = (a.G + a.nchunks - 1) / a.nchunks;
-    a.nchunks = (a.G + a.kcw - 1) / a.kcw;
     a.tiles_m = (a.M + BM - 1) / BM;
     const long blocks = (long)a.tiles_m * ((a.KN + BN - 1) / BN);
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
@@ -175,32 +209,29 @@ hipError_t launch_mfma_tile(ConvArgs a, hipStream_t stream)
     return hipGetLastError();
 }
 
+template <int TYPE, int WM, int WN, int TM, int TN>
+hipError_t launch_mfma_shape(const ConvArgs &a, hipStream_t stream)
+{
+    switch (mfma_chunk_words(a.G)) {
+    case 1: return launch_mfma_tile<TYPE, WM, WN, TM, TN, 1>(a, stream);
+    case 2: return launch_mfma_tile<TYPE, WM, WN, TM, TN, 2>(a, stream);
+    case 3: return launch_mfma_tile<TYPE, WM, WN, TM, TN, 3>(a, stream);
+    default: return launch_mfma_tile<TYPE, WM, WN, TM, TN, 4>(a, stream);
+    }
+}
+
+// shape: 0 = 128x128, 1 = 128x64, 2 = 64x64, 3 = 64x128 (rows x filters per workgroup)
 template <int TYPE>
-hipError_t launch_mfma(const ConvArgs &a, int shape, hipStream_t stream)
+hipError_t launch_mfma_type(const ConvArgs &a, int shape, hipStream_t stream)
 {
     switch (shape) {
-    case 0: return launch_mfma_tile<TYPE, 2, 2, 2, 2, 4>(a, stream);  // 128 x 128
-    case 1: return launch_mfma_tile<TYPE, 4, 1, 1, 2, 4>(a, stream);  // 128 x 64
-    case 2: return launch_mfma_tile<TYPE, 2, 2, 1, 1, 4>(a, stream);  //  64 x 64
-    case 3: return launch_mfma_tile<TYPE, 2, 2, 1, 2, 4>(a, stream);  //  64 x 128
+    case 0: return launch_mfma_shape<TYPE, 2, 2, 2, 2>(a, stream);
+    case 1: return launch_mfma_shape<TYPE, 4, 1, 1, 2>(a, stream);
+    case 2: return launch_mfma_shape<TYPE, 2, 2, 1, 1>(a, stream);
+    case 3: return launch_mfma_shape<TYPE, 2, 2, 1, 2>(a, stream);
     default: return hipErrorInvalidValue;
     }
 }
 
 }  // namespace
-
-bool conv_mfma_exact(const ConvArgs &a) { return (long)a.G * 64 <= (1L << 22); }
-
-hipError_t launch_conv_mfma(int type, const ConvArgs &args, int shape, hipStream_t stream)
-{
-    if (!conv_mfma_exact(args)) return hipErrorInvalidValue;
-    switch (type) {
-    case 0: return launch_mfma<0>(args, shape, stream);
-    case 1: return launch_mfma<1>(args, shape, stream);
-    case 2: return launch_mfma<2>(args, shape, stream);
-    case 3: return launch_mfma<3>(args, shape, stream);
-    default: return hipErrorInvalidValue;
-    }
-}
-
 }  // namespace tab

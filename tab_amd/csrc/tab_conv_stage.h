@@ -77,7 +77,8 @@ struct TileStager {
     __device__ __forceinline__ void init(const ConvArgs &p, int tid, int m0, int n0)
     {
         a_row = tid % BM;
-        a_w0 = tid / BM;
+        // a wave shares its word index when the tile has at least 64 rows: keep the tap decode scalar
+        a_w0 = BM >= 64 ? __builtin_amdgcn_readfirstlane(tid / BM) : tid / BM;
         const int a_m = m0 + a_row;
         a_live = a_m < p.M;
         const int mm = a_live ? a_m : 0;
@@ -88,7 +89,7 @@ struct TileStager {
         iw0 = ow * p.s2 - p.p2;
         a_img = p.qx + (size_t)n * p.H * p.W * p.PC * APL;
         b_row = tid % BN;
-        b_w0 = tid / BN;
+        b_w0 = BN >= 64 ? __builtin_amdgcn_readfirstlane(tid / BN) : tid / BN;
         b_live = (n0 + b_row) < p.KN;
         b_flt = p.qw + (size_t)(b_live ? n0 + b_row : 0) * p.G * BPL;
     }
