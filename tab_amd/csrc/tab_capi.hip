@@ -52,6 +52,10 @@ int check_conv(int type, int p1, int p2, int s1, int s2, int N, int H, int W, in
     if (s->M > kMaxIndex || s->G >= 65536 || s->PC >= 65536 || KW >= 65536 ||
         (long)N * H * W > kMaxIndex || (long)H * W * s->PC * 2 > kMaxIndex)
         return fail(TAB_ERR_BAD_SHAPE, "problem too large for 32-bit row indices (M=%ld, K words=%ld)", s->M, s->G);
+    // a workgroup addresses the images its (at most 256) output pixels touch with 32-bit byte offsets
+    const long image_bytes = (long)H * W * s->PC * s->abits * 8;
+    if (image_bytes * (256 / ((long)s->OH * s->OW) + 2) > 0xffffffffL)
+        return fail(TAB_ERR_BAD_SHAPE, "packed image of %ld bytes is too large for 32-bit offsets", image_bytes);
     return TAB_OK;
 }
 

@@ -24,6 +24,7 @@
 // reads the 32-bit half lane/32 selects of its row (A) or column (B), lane%32.
 #pragma once
 #include "tab_conv_stage.h"
+#include <cstdlib>
 
 namespace tab {
 namespace {
@@ -212,6 +213,7 @@ hipError_t launch_mfma_tile(ConvArgs a, hipStream_t stream)
 template <int TYPE, int WM, int WN, int TM, int TN>
 hipError_t launch_mfma_shape(const ConvArgs &a, hipStream_t stream)
 {
+    if (TYPE != 0 && a.G % 8 == 0 && getenv("TAB_K8")) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 8>(a, stream);
     switch (mfma_chunk_words(a.G)) {
     case 1: return launch_mfma_tile<TYPE, WM, WN, TM, TN, 1>(a, stream);
     case 2: return launch_mfma_tile<TYPE, WM, WN, TM, TN, 2>(a, stream);

@@ -28,17 +28,21 @@ template <int PL> struct Item {
     uint32_t d[2 * PL];
 };
 
+// Buffer descriptor word 3 for untyped 32-bit data on this ISA generation.
+constexpr int kBufferFlags = 0x00020000;
+
+// Loads through a buffer descriptor: an offset at or past the descriptor's size returns zeros, so
+// "this tap is padding", "this row is past M" and "this word is past the end of K" all become one
+// offset select instead of a branch around the load.
 template <int PL>
-__device__ __forceinline__ Item<PL> load_item(const uint64_t *p, bool valid)
+__device__ __forceinline__ Item<PL> load_item(__amdgpu_buffer_rsrc_t rsrc, uint32_t offset)
 {
     Item<PL> it;
     if (PL == 2) {
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (valid) v = *reinterpret_cast<const u32x4 *>(p);
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, offset, 0, 0);
         it.d[0] = v[0]; it.d[1] = v[1]; it.d[2] = v[2]; it.d[3] = v[3];
     } else {
-        u32x2 v = {0u, 0u};
-        if (valid) v = *reinterpret_cast<const u32x2 *>(p);
+        const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, offset, 0, 0);
         it.d[0] = v[0]; it.d[1] = v[1];
     }
     return it;
@@ -54,6 +58,9 @@ __device__ __forceinline__ void store_item(uint32_t *lds, const Item<PL> &it, in
             lds[((pl * Q) + 2 * word + half) * ROWS + row] = it.d[pl * 2 + half];
 }
 
+constexpr uint32_t kNoData = 0xffffffffu;     // activation offset that is always out of range
+constexpr uint32_t kNoFilter = 0x80000000u;   // weight offsets stay below this; adding it leaves the range
+
 template <int TYPE, int BM, int BN, int KCH>
 struct TileStager {
     static constexpr int APL = Planes<TYPE>::A, BPL = Planes<TYPE>::B;
@@ -63,35 +70,46 @@ struct TileStager {
     static constexpr int A_ITEMS = (KCH + A_STEP - 1) / A_STEP, B_ITEMS = (KCH + B_STEP - 1) / B_STEP;
     static_assert(kConvThreads % BM == 0 && kConvThreads % BN == 0, "tile rows must divide the workgroup");
 
-    // A: this thread fetches words (a_w0 + i*A_STEP) of output pixel m0 + a_row
+    // A: this thread fetches words (a_w0 + i*A_STEP) of output pixel m0 + a_row.  a_base is the
+    // byte offset of input pixel (ih0, iw0) from the first image the tile touches, in wrapping
+    // 32-bit arithmetic (the pixel itself may lie in the padding).
+    __amdgpu_buffer_rsrc_t a_rsrc, b_rsrc;
     int a_row, a_w0, ih0, iw0;
-    bool a_live;
-    const uint64_t *a_img;
+    uint32_t a_base;
     // B: this thread fetches words (b_w0 + i*B_STEP) of filter n0 + b_row
     int b_row, b_w0;
-    bool b_live;
-    const uint64_t *b_flt;
+    uint32_t b_base;
     Item<APL> a_reg[A_ITEMS];
     Item<BPL> b_reg[B_ITEMS];
 
     __device__ __forceinline__ void init(const ConvArgs &p, int tid, int m0, int n0)
     {
         a_row = tid % BM;
-        // a wave shares its word index when the tile has at least 64 rows: keep the tap decode scalar
+        // a wave shares its word index when the tile has at least 64 rows: the tap decode stays scalar
         a_w0 = BM >= 64 ? __builtin_amdgcn_readfirstlane(tid / BM) : tid / BM;
+        const int pixels = p.OH * p.OW;
+        const int n_first = m0 / pixels;  // uniform
+        const size_t image_words = (size_t)p.H * p.W * p.PC * APL;
+        const size_t a_bytes = (size_t)(p.N - n_first) * image_words * 8;
+        a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(p.qx + (size_t)n_first * image_words), 0,
+                                                   a_bytes > 0xffffffffull ? (int)0xffffffffu : (int)a_bytes, kBufferFlags);
         const int a_m = m0 + a_row;
-        a_live = a_m < p.M;
-        const int mm = a_live ? a_m : 0;
-        const int n = mm / (p.OH * p.OW);
-        const int r = mm - n * (p.OH * p.OW);
+        const bool a_live = a_m < p.M;
+        const int mm = a_live ? a_m : m0;
+        const int n = mm / pixels;
+        const int r = mm - n * pixels;
         const int oh = r / p.OW, ow = r - oh * p.OW;
-        ih0 = oh * p.s1 - p.p1;
+        ih0 = a_live ? oh * p.s1 - p.p1 : -(1 << 30);  // a dead row fails every bounds check
         iw0 = ow * p.s2 - p.p2;
-        a_img = p.qx + (size_t)n * p.H * p.W * p.PC * APL;
+        a_base = (uint32_t)((((n - n_first) * p.H + (oh * p.s1 - p.p1)) * p.W + iw0) * p.PC) * (uint32_t)(APL * 8);
+
         b_row = tid % BN;
         b_w0 = BN >= 64 ? __builtin_amdgcn_readfirstlane(tid / BN) : tid / BN;
-        b_live = (n0 + b_row) < p.KN;
-        b_flt = p.qw + (size_t)(b_live ? n0 + b_row : 0) * p.G * BPL;
+        const size_t filter_bytes = (size_t)p.G * BPL * 8;
+        const size_t b_bytes = (size_t)(p.KN - n0) * filter_bytes;
+        b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(p.qw + (size_t)n0 * p.G * BPL), 0,
+                                                   b_bytes > kNoFilter ? (int)kNoFilter : (int)b_bytes, kBufferFlags);
+        b_base = (n0 + b_row) < p.KN ? (uint32_t)b_row * (uint32_t)filter_bytes : kNoFilter;
     }
 
     // issue the global loads of one chunk into registers
@@ -102,23 +120,21 @@ struct TileStager {
         for (int i = 0; i < A_ITEMS; i++) {
             const int w = a_w0 + i * A_STEP;
             const int g = g0 + w;
-            // g is uniform over the wave when BM >= 64; the tap decode is a few multiplies
             const uint32_t tap = fastdiv((uint32_t)g, p.div_pc);
             const int pc = g - (int)tap * p.PC;
-            const uint32_t kh = fastdiv(tap, p.div_kw);
+            uint32_t kh = fastdiv(tap, p.div_kw);
             const int kw = (int)tap - (int)kh * p.KW;
-            const int ih = ih0 + (int)kh, iw = iw0 + kw;
-            const bool ok = a_live && w < p.kcw && g < p.G && (unsigned)ih < (unsigned)p.H &&
-                            (unsigned)iw < (unsigned)p.W;
-            const size_t off = ok ? ((size_t)(ih * p.W + iw) * p.PC + pc) * APL : 0;
-            a_reg[i] = load_item<APL>(a_img + off, ok);
+            if (w >= p.kcw || g >= p.G) kh = 1u << 29;  // past the chunk or past K: no row is in range
+            const uint32_t tap_off = (uint32_t)(((int)kh * p.W + kw) * p.PC + pc) * (uint32_t)(APL * 8);
+            const bool ok = (unsigned)(ih0 + (int)kh) < (unsigned)p.H && (unsigned)(iw0 + kw) < (unsigned)p.W;
+            a_reg[i] = load_item<APL>(a_rsrc, ok ? a_base + tap_off : kNoData);
         }
 #pragma unroll
         for (int i = 0; i < B_ITEMS; i++) {
             const int w = b_w0 + i * B_STEP;
             const int g = g0 + w;
-            const bool ok = b_live && w < p.kcw && g < p.G;
-            b_reg[i] = load_item<BPL>(b_flt + (ok ? (size_t)g * BPL : 0), ok);
+            const uint32_t word_off = (w < p.kcw && g < p.G) ? (uint32_t)g * (uint32_t)(BPL * 8) : kNoFilter;
+            b_reg[i] = load_item<BPL>(b_rsrc, b_base + word_off);
         }
     }
 
