@@ -24,7 +24,7 @@
 // reads the 32-bit half lane/32 selects of its row (A) or column (B), lane%32.
 #pragma once
 #include "tab_conv_stage.h"
-#include <cstdlib>
+#include <type_traits>
 
 namespace tab {
 namespace {
@@ -75,13 +75,14 @@ __device__ __forceinline__ i32x8 expand_ternary(uint32_t s, uint32_t z)
     return r;
 }
 
-template <int TYPE, int WM, int WN, int TM, int TN, int KCH>
+template <int TYPE, int WM, int WN, int TM, int TN, int KCH, bool INTAP>
 __global__ __launch_bounds__(kConvThreads) void conv_mfma(const ConvArgs p)
 {
     static_assert(WM * WN * 64 == kConvThreads, "four waves");
     constexpr int APL = Planes<TYPE>::A, BPL = Planes<TYPE>::B;
     constexpr int BM = 32 * WM * TM, BN = 32 * WN * TN;
-    using Stager = TileStager<TYPE, BM, BN, KCH>;
+    using Stager = typename std::conditional<INTAP, TapStager<TYPE, BM, BN, INTAP ? KCH : 2>, TileStager<TYPE, BM, BN, KCH>>::type;
+    constexpr int A_STRIDE = Stager::A_STRIDE, B_STRIDE = Stager::B_STRIDE;
     constexpr int Q = Stager::Q, A_DWORDS = Stager::A_DWORDS, B_DWORDS = Stager::B_DWORDS;
 
     __shared__ __attribute__((aligned(16))) uint32_t lds[2 * (A_DWORDS + B_DWORDS)];
@@ -127,11 +128,11 @@ __global__ __launch_bounds__(kConvThreads) void conv_mfma(const ConvArgs p)
 #pragma unroll
             for (int pl = 0; pl < APL; pl++)
 #pragma unroll
-                for (int mt = 0; mt < TM; mt++) a_w[w][pl][mt] = la[(pl * Q + q) * BM + mt * 32];
+                for (int mt = 0; mt < TM; mt++) a_w[w][pl][mt] = la[(pl * Q + q) * A_STRIDE + mt * 32];
 #pragma unroll
             for (int pl = 0; pl < BPL; pl++)
 #pragma unroll
-                for (int nt = 0; nt < TN; nt++) b_w[w][pl][nt] = lb[(pl * Q + q) * BN + nt * 32];
+                for (int nt = 0; nt < TN; nt++) b_w[w][pl][nt] = lb[(pl * Q + q) * B_STRIDE + nt * 32];
         };
         read_word(0);
 #pragma unroll
@@ -197,7 +198,7 @@ inline int mfma_chunk_words(int G)
     return best;
 }
 
-template <int TYPE, int WM, int WN, int TM, int TN, int KCH>
+template <int TYPE, int WM, int WN, int TM, int TN, int KCH, bool INTAP>
 hipError_t launch_mfma_tile(ConvArgs a, hipStream_t stream)
 {
     constexpr int BM = 32 * WM * TM, BN = 32 * WN * TN;
@@ -206,19 +207,21 @@ hipError_t launch_mfma_tile(ConvArgs a, hipStream_t stream)
     a.tiles_m = (a.M + BM - 1) / BM;
     const long blocks = (long)a.tiles_m * ((a.KN + BN - 1) / BN);
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
-    conv_mfma<TYPE, WM, WN, TM, TN, KCH><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
+    conv_mfma<TYPE, WM, WN, TM, TN, KCH, INTAP><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
     return hipGetLastError();
 }
 
 template <int TYPE, int WM, int WN, int TM, int TN>
 hipError_t launch_mfma_shape(const ConvArgs &a, hipStream_t stream)
 {
-    if (TYPE != 0 && a.G % 8 == 0 && getenv("TAB_K8")) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 8>(a, stream);
+    // chunks that stay inside one tap take the piece stager
+    if (a.PC % 4 == 0) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 4, true>(a, stream);
+    if (a.PC % 2 == 0) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 2, true>(a, stream);
     switch (mfma_chunk_words(a.G)) {
-    case 1: return launch_mfma_tile<TYPE, WM, WN, TM, TN, 1>(a, stream);
-    case 2: return launch_mfma_tile<TYPE, WM, WN, TM, TN, 2>(a, stream);
-    case 3: return launch_mfma_tile<TYPE, WM, WN, TM, TN, 3>(a, stream);
-    default: return launch_mfma_tile<TYPE, WM, WN, TM, TN, 4>(a, stream);
+    case 1: return launch_mfma_tile<TYPE, WM, WN, TM, TN, 1, false>(a, stream);
+    case 2: return launch_mfma_tile<TYPE, WM, WN, TM, TN, 2, false>(a, stream);
+    case 3: return launch_mfma_tile<TYPE, WM, WN, TM, TN, 3, false>(a, stream);
+    default: return launch_mfma_tile<TYPE, WM, WN, TM, TN, 4, false>(a, stream);
     }
 }
 

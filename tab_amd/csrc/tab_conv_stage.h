@@ -65,6 +65,7 @@ template <int TYPE, int BM, int BN, int KCH>
 struct TileStager {
     static constexpr int APL = Planes<TYPE>::A, BPL = Planes<TYPE>::B;
     static constexpr int Q = 2 * KCH;  // 32-bit k-slices per chunk
+    static constexpr int A_STRIDE = BM, B_STRIDE = BN;  // dwords between consecutive k-slices
     static constexpr int A_DWORDS = APL * Q * BM, B_DWORDS = BPL * Q * BN;
     static constexpr int A_STEP = kConvThreads / BM, B_STEP = kConvThreads / BN;  // words per pass over the rows
     static constexpr int A_ITEMS = (KCH + A_STEP - 1) / A_STEP, B_ITEMS = (KCH + B_STEP - 1) / B_STEP;
@@ -152,6 +153,115 @@ struct TileStager {
             const int w = b_w0 + i * B_STEP;
             if (w < KCH) store_item<BPL, BN, Q>(lb, b_reg[i], w, b_row);
         }
+    }
+};
+
+// Stager for the case where a chunk never leaves a filter tap (PC % KCH == 0, KCH even): the tap
+// decode is one scalar computation per chunk, and threads fetch 16-byte pieces (two words of a
+// one-plane operand, one word of a two-plane operand) with the pieces of a row on neighbouring
+// lanes, so that one load instruction covers whole runs of the row's K-contiguous memory instead
+// of 8 bytes from each of 64 rows.  LDS layout as in TileStager, but k-slices are ROWS + 8
+// dwords apart so that the pieces of one store instruction fall into different banks.
+template <int TYPE, int BM, int BN, int KCH>
+struct TapStager {
+    static constexpr int APL = Planes<TYPE>::A, BPL = Planes<TYPE>::B;
+    static constexpr int Q = 2 * KCH;
+    static constexpr int A_STRIDE = BM + 8, B_STRIDE = BN + 8;
+    static constexpr int A_DWORDS = APL * Q * A_STRIDE, B_DWORDS = BPL * Q * B_STRIDE;
+    static constexpr int PA = KCH * APL / 2, PB = KCH * BPL / 2;  // 16-byte pieces per row and chunk
+    static constexpr int A_ITEMS = (BM * PA + kConvThreads - 1) / kConvThreads;
+    static constexpr int B_ITEMS = (BN * PB + kConvThreads - 1) / kConvThreads;
+    static_assert(KCH % 2 == 0, "pieces pair the words of one-plane operands");
+
+    __amdgpu_buffer_rsrc_t a_rsrc, b_rsrc;
+    int ih0[A_ITEMS], iw0[A_ITEMS];
+    uint32_t a_base[A_ITEMS], b_base[B_ITEMS];  // byte offsets, piece included
+    int a_lds[A_ITEMS], b_lds[B_ITEMS];         // dword index of the piece's first slice; < 0: no piece
+    u32x4 a_reg[A_ITEMS], b_reg[B_ITEMS];
+
+    template <int PL, int P, int STRIDE>
+    static __device__ __forceinline__ int lds_index(int row, int piece)
+    {
+        // one-plane: piece = words 2*piece, 2*piece+1 -> slices 4*piece..; two-plane: piece = word
+        return (PL == 1 ? 4 * piece : 2 * piece) * STRIDE + row;
+    }
+
+    __device__ __forceinline__ void init(const ConvArgs &p, int tid, int m0, int n0)
+    {
+        const int pixels = p.OH * p.OW;
+        const int n_first = m0 / pixels;  // uniform
+        const size_t image_words = (size_t)p.H * p.W * p.PC * APL;
+        const size_t a_bytes = (size_t)(p.N - n_first) * image_words * 8;
+        a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(p.qx + (size_t)n_first * image_words), 0,
+                                                   a_bytes > 0xffffffffull ? (int)0xffffffffu : (int)a_bytes, kBufferFlags);
+#pragma unroll
+        for (int i = 0; i < A_ITEMS; i++) {
+            const int idx = tid + i * kConvThreads;
+            const int row = idx / PA, piece = idx % PA;
+            const int a_m = m0 + row;
+            const bool live = row < BM && a_m < p.M;
+            const int mm = live ? a_m : m0;
+            const int n = mm / pixels;
+            const int r = mm - n * pixels;
+            const int oh = r / p.OW, ow = r - oh * p.OW;
+            ih0[i] = live ? oh * p.s1 - p.p1 : -(1 << 30);  // a dead row fails every bounds check
+            iw0[i] = ow * p.s2 - p.p2;
+            a_base[i] = (uint32_t)((((n - n_first) * p.H + (oh * p.s1 - p.p1)) * p.W + iw0[i]) * p.PC) * (uint32_t)(APL * 8) +
+                        (uint32_t)piece * 16u;
+            a_lds[i] = row < BM ? lds_index<APL, PA, A_STRIDE>(row, piece) : -1;
+        }
+        const size_t filter_bytes = (size_t)p.G * BPL * 8;
+        const size_t b_bytes = (size_t)(p.KN - n0) * filter_bytes;
+        b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(p.qw + (size_t)n0 * p.G * BPL), 0,
+                                                   b_bytes > kNoFilter ? (int)kNoFilter : (int)b_bytes, kBufferFlags);
+#pragma unroll
+        for (int i = 0; i < B_ITEMS; i++) {
+            const int idx = tid + i * kConvThreads;
+            const int row = idx / PB, piece = idx % PB;
+            const bool live = row < BN && (n0 + row) < p.KN;
+            b_base[i] = live ? (uint32_t)row * (uint32_t)filter_bytes + (uint32_t)piece * 16u : kNoFilter;
+            b_lds[i] = row < BN ? lds_index<BPL, PB, B_STRIDE>(row, piece) : -1;
+        }
+    }
+
+    __device__ __forceinline__ void fetch(const ConvArgs &p, int chunk)
+    {
+        const int g0 = chunk * KCH;  // first word of the chunk; the whole chunk lies in one tap
+        const uint32_t tap = fastdiv((uint32_t)g0, p.div_pc);
+        const int pc = g0 - (int)tap * p.PC;
+        const int kh = (int)fastdiv(tap, p.div_kw);
+        const int kw = (int)tap - kh * p.KW;
+        const uint32_t tap_off = (uint32_t)((kh * p.W + kw) * p.PC + pc) * (uint32_t)(APL * 8);
+#pragma unroll
+        for (int i = 0; i < A_ITEMS; i++) {
+            const bool ok = (unsigned)(ih0[i] + kh) < (unsigned)p.H && (unsigned)(iw0[i] + kw) < (unsigned)p.W;
+            a_reg[i] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, ok ? a_base[i] + tap_off : kNoData, 0, 0);
+        }
+        const uint32_t word_off = (uint32_t)g0 * (uint32_t)(BPL * 8);
+#pragma unroll
+        for (int i = 0; i < B_ITEMS; i++)
+            b_reg[i] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, b_base[i] + word_off, 0, 0);
+    }
+
+    template <int PL, int STRIDE>
+    static __device__ __forceinline__ void store_piece(uint32_t *lds, int index, const u32x4 &v)
+    {
+        if (index < 0) return;
+        if (PL == 1) {  // (word, half) = (0,0) (0,1) (1,0) (1,1): four consecutive slices
+#pragma unroll
+            for (int j = 0; j < 4; j++) lds[index + j * STRIDE] = v[j];
+        } else {        // (plane, half): slices 2w, 2w+1 of plane 0, then of plane 1
+#pragma unroll
+            for (int j = 0; j < 4; j++) lds[index + ((j >> 1) * Q + (j & 1)) * STRIDE] = v[j];
+        }
+    }
+
+    __device__ __forceinline__ void stage(uint32_t *buf) const
+    {
+#pragma unroll
+        for (int i = 0; i < A_ITEMS; i++) store_piece<APL, A_STRIDE>(buf, a_lds[i], a_reg[i]);
+#pragma unroll
+        for (int i = 0; i < B_ITEMS; i++) store_piece<BPL, B_STRIDE>(buf + A_DWORDS, b_lds[i], b_reg[i]);
     }
 };
 
