@@ -113,6 +113,20 @@ int tab_conv2d_packed(const int64_t *dev_QX, const int64_t *dev_QW, const int32_
                       int type, int padding1, int padding2, int stride1, int stride2, int N,
                       int H, int W, int C, int KN, int KH, int KW, float *dev_Y, void *stream);
 
+/*
+ * Which kernel tab_conv2d / tab_conv2d_packed launch.  Both give bit-identical Y; the switch exists
+ * for verification and tuning and has no counterpart in the reference (which has one GEMM kernel
+ * per type, TAB_GEMM.cu:25-147).  Process-wide, not thread-safe against concurrent conv calls.
+ *   TAB_CONV_AUTO      (tile -1) the library's choice: matrix cores, tile picked from the shape
+ *   TAB_CONV_MATRIX    bit planes expanded to FP4 operands of v_mfma_f32_32x32x64_f8f6f4;
+ *                      tile 0: 128x128, 1: 128x64, 2: 64x64, 3: 32x32 with K split over the
+ *                      four waves; -1: picked from the shape
+ *   TAB_CONV_POPCOUNT  the reference's xor/and + popcount formulation on the vector ALU;
+ *                      tile 0: big, 1: medium, 2: small; -1: picked from the shape
+ */
+enum { TAB_CONV_AUTO = 0, TAB_CONV_MATRIX = 1, TAB_CONV_POPCOUNT = 2 };
+int tab_set_conv_kernel(int kernel, int tile);
+
 #ifdef __cplusplus
 }
 #endif

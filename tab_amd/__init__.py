@@ -168,9 +168,19 @@ def Conv2dPacked(QX, QW, btn, type, padding1, padding2, stride1, stride2, N, H, 
     return Y
 
 
+CONV_AUTO, CONV_MATRIX, CONV_POPCOUNT = 0, 1, 2
+
+
+def set_conv_kernel(kernel=CONV_AUTO, tile=-1):
+    """Pick the conv kernel (process-wide): CONV_AUTO, CONV_MATRIX (tile 0..3 or -1) or
+    CONV_POPCOUNT (tile 0..2 or -1).  Every choice gives bit-identical outputs."""
+    _capi.check(_lib, _lib.tab_set_conv_kernel(int(kernel), int(tile)))
+
+
 # names of the reference's CPU module (TAB_CPU.cpp:636-639)
 TAB_Quantize = Quantize
 TAB_Conv2d = Conv2d
 
 __all__ = ["Quantize", "Conv2d", "Conv2dPacked", "Threshold", "TAB_Quantize", "TAB_Conv2d", "TabError",
-           "packed_channels", "out_shape", "version", "TNN", "TBN", "BTN", "BNN"]
+           "packed_channels", "out_shape", "version", "TNN", "TBN", "BTN", "BNN", "set_conv_kernel",
+           "CONV_AUTO", "CONV_MATRIX", "CONV_POPCOUNT"]

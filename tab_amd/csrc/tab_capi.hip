@@ -82,6 +82,16 @@ const char *tab_version(void) { return "tab_amd 0.1 gfx950"; }
 /* Tuning hook for benchmarking scripts; deliberately absent from include/tab_amd.h. */
 void tab_internal_force_conv_tile(int tm, int ng) { tab::force_conv_tile(tm, ng); }
 
+int tab_set_conv_kernel(int kernel, int tile)
+{
+    static const int popcount_tm[4] = {7, 8, 4, 2};  // 7: the popcount kernel's own choice
+    if (kernel == TAB_CONV_AUTO && tile == -1) tab::force_conv_tile(0, 0);
+    else if (kernel == TAB_CONV_MATRIX && tile >= -1 && tile <= 3) tab::force_conv_tile(9, tile);
+    else if (kernel == TAB_CONV_POPCOUNT && tile >= -1 && tile <= 2) tab::force_conv_tile(popcount_tm[tile + 1], 0);
+    else return fail(TAB_ERR_BAD_ARGUMENT, "no conv kernel %d with tile %d", kernel, tile);
+    return TAB_OK;
+}
+
 int tab_packed_channels(int C) { return (C + tab::kWordBits - 1) / tab::kWordBits; }
 
 int tab_out_extent(int in, int pad, int k, int stride)

@@ -314,11 +314,9 @@ template <int TYPE>
 hipError_t launch_type(const ConvArgs &a, hipStream_t stream)
 {
     constexpr int BIG_BN = (TYPE == 0) ? 64 : 128;
-    if (g_force_tm) {
-        if (g_force_tm == 8) return launch_big<TYPE>(a, stream);
-        if (g_force_tm == 4) return launch_tile<TYPE, 4, 1, 4, true>(a, stream);
-        return launch_tile<TYPE, 2, 1, 8, true>(a, stream);
-    }
+    if (g_force_tm == 8) return launch_big<TYPE>(a, stream);
+    if (g_force_tm == 4) return launch_tile<TYPE, 4, 1, 4, true>(a, stream);
+    if (g_force_tm == 2) return launch_tile<TYPE, 2, 1, 8, true>(a, stream);
     auto tiles = [&](int bm, int bn) { return (long)((a.M + bm - 1) / bm) * ((a.KN + bn - 1) / bn); };
     if (a.KN > BIG_BN / 2 && tiles(128, BIG_BN) >= 3072) return launch_big<TYPE>(a, stream);
     if (tiles(64, 64) >= 512) return launch_tile<TYPE, 4, 1, 4, true>(a, stream);
@@ -347,9 +345,24 @@ hipError_t launch_conv_mfma(int type, const ConvArgs &args, int shape, hipStream
     }
 }
 
+// Workgroup tile of the matrix-core kernel, from measurements over the ResNet-18 and sweep layers at
+// N = 16 and N = 256: the largest tile that still gives the chip about four workgroups per CU; below
+// roughly 200 workgroups of 64x64 the launch is latency-bound and the k-split 32x32 shape wins.
+int conv_mfma_shape(const ConvArgs &a)
+{
+    auto tiles = [&](int bm, int bn) { return (long)((a.M + bm - 1) / bm) * ((a.KN + bn - 1) / bn); };
+    if (a.KN > 64 && tiles(128, 128) >= 1024) return 0;
+    if (tiles(128, 64) >= 1024) return 1;
+    if (tiles(64, 64) >= 192) return 2;
+    return 3;
+}
+
 hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream)
 {
-    if (g_force_tm == 9) return launch_conv_mfma(type, args, g_force_ng, stream);
+    if (g_force_tm == 9) return launch_conv_mfma(type, args, g_force_ng < 0 ? conv_mfma_shape(args) : g_force_ng, stream);
+    // default path: matrix cores; the popcount kernel takes over when K is too long for exact fp32
+    // accumulation (and when a benchmark forces one of its tiles)
+    if (g_force_tm == 0 && conv_mfma_exact(args)) return launch_conv_mfma(type, args, conv_mfma_shape(args), stream);
     switch (type) {
     case 0: return launch_type<0>(args, stream);
     case 1: return launch_type<1>(args, stream);

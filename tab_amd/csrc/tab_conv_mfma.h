@@ -75,10 +75,12 @@ __device__ __forceinline__ i32x8 expand_ternary(uint32_t s, uint32_t z)
     return r;
 }
 
-template <int TYPE, int WM, int WN, int TM, int TN, int KCH, bool INTAP>
+template <int TYPE, int WM, int WN, int TM, int TN, int KCH, bool INTAP, int KS = 1>
 __global__ __launch_bounds__(kConvThreads) void conv_mfma(const ConvArgs p)
 {
-    static_assert(WM * WN * 64 == kConvThreads, "four waves");
+    static_assert(WM * WN * KS * 64 == kConvThreads, "four waves");
+    static_assert(KCH % KS == 0 && (KS == 1 || (TM == 1 && TN == 1)), "k-split waves share one 32x32 tile");
+    constexpr int WPW = KCH / KS;  // words of a chunk each wave multiplies
     constexpr int APL = Planes<TYPE>::A, BPL = Planes<TYPE>::B;
     constexpr int BM = 32 * WM * TM, BN = 32 * WN * TN;
     using Stager = typename std::conditional<INTAP, TapStager<TYPE, BM, BN, INTAP ? KCH : 2>, TileStager<TYPE, BM, BN, KCH>>::type;
@@ -86,12 +88,14 @@ __global__ __launch_bounds__(kConvThreads) void conv_mfma(const ConvArgs p)
     constexpr int Q = Stager::Q, A_DWORDS = Stager::A_DWORDS, B_DWORDS = Stager::B_DWORDS;
 
     __shared__ __attribute__((aligned(16))) uint32_t lds[2 * (A_DWORDS + B_DWORDS)];
+    __shared__ float partial[KS > 1 ? KS * 17 * 64 : 1];  // k-split: 16 accumulators + the BTN count per lane
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int r = lane & 31;   // row of an A tile / column of a B tile
     const int kb = lane >> 5;  // which 32-bit half of the word this lane feeds
-    const int wm = wave % WM, wn = wave / WM;
+    const int ks = wave / (WM * WN);  // which words of every chunk this wave takes
+    const int wm = (wave % (WM * WN)) % WM, wn = (wave % (WM * WN)) / WM;
     const int tile_m = blockIdx.x % p.tiles_m, tile_n = blockIdx.x / p.tiles_m;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
@@ -122,9 +126,9 @@ __global__ __launch_bounds__(kConvThreads) void conv_mfma(const ConvArgs p)
         // nothing for a ternary operand and +64 per word for binary x binary (the BNN bias below
         // counts them).  LDS reads run one word ahead of the matrix cores.
         const uint32_t *la = lds + (chunk & 1) * (A_DWORDS + B_DWORDS) + a_off, *lb = la - a_off + A_DWORDS + b_off;
-        uint32_t a_w[KCH][APL][TM], b_w[KCH][BPL][TN];
+        uint32_t a_w[WPW][APL][TM], b_w[WPW][BPL][TN];
         auto read_word = [&](int w) {
-            const int q = 2 * w + kb;
+            const int q = 2 * (ks + KS * w) + kb;
 #pragma unroll
             for (int pl = 0; pl < APL; pl++)
 #pragma unroll
@@ -136,8 +140,8 @@ __global__ __launch_bounds__(kConvThreads) void conv_mfma(const ConvArgs p)
         };
         read_word(0);
 #pragma unroll
-        for (int w = 0; w < KCH; w++) {
-            if (w + 1 < KCH) read_word(w + 1);
+        for (int w = 0; w < WPW; w++) {
+            if (w + 1 < WPW) read_word(w + 1);
             i32x8 af[TM], bf[TN];
 #pragma unroll
             for (int mt = 0; mt < TM; mt++)
@@ -161,6 +165,33 @@ __global__ __launch_bounds__(kConvThreads) void conv_mfma(const ConvArgs p)
     // ---- epilogue: accumulator element 4*j + i of lane (kb, r) is C[8*j + 4*kb + i][r] -------
     const int wave_m0 = m0 + wm * (32 * TM), wave_n0 = n0 + wn * (32 * TN);
     const bool whole = wave_m0 + 32 * TM <= p.M && wave_n0 + 32 * TN <= p.KN;  // wave-uniform
+    if (KS > 1) {
+        // the KS waves hold partial sums of the same tile: exchange them through LDS; wave ks
+        // finishes rows 8*ks .. 8*ks+7
+#pragma unroll
+        for (int e = 0; e < 16; e++) partial[(ks * 17 + e) * 64 + lane] = acc[0][0][e];
+        partial[(ks * 17 + 16) * 64 + lane] = (float)b_nonzero[0];
+        __syncthreads();
+        float sum[5];
+#pragma unroll
+        for (int e = 0; e < 5; e++) {
+            sum[e] = 0.f;
+            const int src = e < 4 ? 4 * ks + e : 16;
+#pragma unroll
+            for (int k = 0; k < KS; k++) sum[e] += partial[(k * 17 + src) * 64 + lane];
+        }
+        const int col = wave_n0 + r;
+        const bool col_ok = col < p.KN;
+        float bias = 0.f;
+        if (TYPE == 2) bias = (float)(col_ok ? p.btn[col] : 0) - (sum[4] + __shfl_xor(sum[4], 32, 64));
+        if (TYPE == 3) bias = (float)(p.num - 64 * p.nchunks * KCH);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int m = wave_m0 + 8 * ks + 4 * kb + i;
+            if (col_ok && m < p.M) p.y[(size_t)m * p.KN + col] = sum[i] + bias;
+        }
+        return;
+    }
 #pragma unroll
     for (int nt = 0; nt < TN; nt++) {
         const int col = wave_n0 + nt * 32 + r;
@@ -198,7 +229,7 @@ inline int mfma_chunk_words(int G)
     return best;
 }
 
-template <int TYPE, int WM, int WN, int TM, int TN, int KCH, bool INTAP>
+template <int TYPE, int WM, int WN, int TM, int TN, int KCH, bool INTAP, int KS = 1>
 hipError_t launch_mfma_tile(ConvArgs a, hipStream_t stream)
 {
     constexpr int BM = 32 * WM * TM, BN = 32 * WN * TN;
@@ -207,7 +238,7 @@ hipError_t launch_mfma_tile(ConvArgs a, hipStream_t stream)
     a.tiles_m = (a.M + BM - 1) / BM;
     const long blocks = (long)a.tiles_m * ((a.KN + BN - 1) / BN);
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
-    conv_mfma<TYPE, WM, WN, TM, TN, KCH, INTAP><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
+    conv_mfma<TYPE, WM, WN, TM, TN, KCH, INTAP, KS><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
     return hipGetLastError();
 }
 
@@ -225,7 +256,8 @@ hipError_t launch_mfma_shape(const ConvArgs &a, hipStream_t stream)
     }
 }
 
-// shape: 0 = 128x128, 1 = 128x64, 2 = 64x64, 3 = 64x128 (rows x filters per workgroup)
+// shape: 0 = 128x128, 1 = 128x64, 2 = 64x64 (rows x filters per workgroup), 3 = 32x32 with the four
+// waves splitting every chunk of four words between them
 template <int TYPE>
 hipError_t launch_mfma_type(const ConvArgs &a, int shape, hipStream_t stream)
 {
@@ -233,7 +265,9 @@ hipError_t launch_mfma_type(const ConvArgs &a, int shape, hipStream_t stream)
     case 0: return launch_mfma_shape<TYPE, 2, 2, 2, 2>(a, stream);
     case 1: return launch_mfma_shape<TYPE, 4, 1, 1, 2>(a, stream);
     case 2: return launch_mfma_shape<TYPE, 2, 2, 1, 1>(a, stream);
-    case 3: return launch_mfma_shape<TYPE, 2, 2, 1, 2>(a, stream);
+    case 3:
+        if (a.PC % 4 == 0) return launch_mfma_tile<TYPE, 1, 1, 1, 1, 4, true, 4>(a, stream);
+        return launch_mfma_tile<TYPE, 1, 1, 1, 1, 4, false, 4>(a, stream);
     default: return hipErrorInvalidValue;
     }
 }

@@ -89,6 +89,58 @@ def test_large_channel_layers(type, case):
     _conv_case(type, *case)
 
 
+KERNEL_VARIANTS = [(tab_amd.CONV_MATRIX, t) for t in range(4)] + [(tab_amd.CONV_POPCOUNT, t) for t in range(3)]
+VARIANT_CASES = [
+    (2, 9, 6, 70, 5, 3, 3, 1, 0, 1, 2),        # one word per pixel pair: chunks cross taps
+    (2, 12, 12, 192, 130, 3, 3, 1, 1, 1, 1),   # PC = 3: odd words per tap
+    (3, 10, 10, 128, 40, 3, 3, 1, 1, 1, 1),    # PC = 2: chunks of two words inside a tap
+    (2, 9, 9, 512, 72, 3, 3, 1, 1, 2, 2),      # PC = 8: chunks of four words inside a tap
+    (1, 3, 3, 8192, 12, 3, 3, 1, 1, 1, 1),     # K = 73728 bits
+]
+
+
+@pytest.fixture
+def restore_kernel_choice():
+    yield
+    tab_amd.set_conv_kernel(tab_amd.CONV_AUTO, -1)
+
+
+@pytest.mark.parametrize("variant", KERNEL_VARIANTS)
+@pytest.mark.parametrize("type", [0, 1, 2, 3])
+def test_every_kernel_variant(type, variant, restore_kernel_choice):
+    """Each selectable kernel and tile shape against the oracle, on shapes that take every staging
+    path (chunks inside a tap / across taps, ragged M, KN and C)."""
+    tab_amd.set_conv_kernel(*variant)
+    for case in VARIANT_CASES:
+        _conv_case(type, *case, seed=11 + type, relu=(type == 1))
+
+
+def test_kernel_variants_agree_on_random_bits(restore_kernel_choice):
+    """Arbitrary 64-bit patterns in QW and btn (sign bits outside the nonzero plane, tail bits set):
+    every kernel follows the reference's formulas, so all of them agree with the oracle."""
+    N, H, W, C, KN, KH, KW = 2, 6, 6, 256, 40, 3, 3
+    rng = np.random.default_rng(5)
+    x, x_ths, _, _ = make_layer(0, N, H, W, C, KN, KH, KW, seed=4)
+    for type in range(4):
+        qw = rng.integers(-2**63, 2**63 - 1, size=(KN, KH, KW, C // 64, weight_bits(type)), dtype=np.int64, endpoint=True)
+        btn = rng.integers(0, 1000, size=KN).astype(np.int32)
+        ths = x_ths if act_bits(type) == 2 else torch.zeros(N)
+        want = oracle.conv2d(x.numpy(), qw, ths.numpy(), btn, type, 1, 1, 1, 1, N, H, W, C, KN, KH, KW)
+        for variant in KERNEL_VARIANTS:
+            print(f"[case] random QW bits type={type} kernel={variant}", flush=True)
+            tab_amd.set_conv_kernel(*variant)
+            y = tab_amd.Conv2d(x.cuda(), torch.from_numpy(qw).cuda(), ths.cuda(), torch.from_numpy(btn).cuda(),
+                               type, 1, 1, 1, 1, N, H, W, C, KN, KH, KW)
+            assert np.array_equal(y.cpu().numpy(), want), f"type {type} kernel {variant}"
+
+
+def test_set_conv_kernel_rejects_unknown():
+    with pytest.raises(tab_amd.TabError, match="no conv kernel"):
+        tab_amd.set_conv_kernel(5, 0)
+    with pytest.raises(tab_amd.TabError, match="no conv kernel"):
+        tab_amd.set_conv_kernel(tab_amd.CONV_MATRIX, 9)
+
+
 def test_arbitrary_weight_bit_patterns():
     """QW is caller data: the kernels must follow the formulas for any 64-bit pattern, including
     sign bits outside the nonzero plane (the notebook passes a 1-bit QW to the 2-bit types)."""
