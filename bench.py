@@ -20,10 +20,15 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 TYPE_NAMES = {0: "TNN", 1: "TBN", 2: "BTN", 3: "BNN"}
-# VALU popcount roofline.  A SIMD issues one wave64 VALU instruction in `cycles`:
-# measured on MI355X with tab_amd/lib/valu_peak (profiles/valu_issue_rates.txt): 2 cycles for
-# v_xor/v_and/v_bitop3 (128 lanes/clk/CU) and 4 cycles for v_bcnt_u32_b32 (64 lanes/clk/CU).
-# Per 32-bit word pair (= 64 binary ops per lane) the kernels issue
+# Matrix-core roofline of the default conv kernel: the bit planes are multiplied as FP4 (E2M1)
+# operands of v_mfma_f32_32x32x64_f8f6f4; MI355X's published dense FP4 rate is 10.1 PFLOP/s, and
+# one effective binary op (half a multiply-accumulate) is one such flop.
+MFMA_FP4_PEAK_TOPS = 10100.0
+# VALU popcount roofline, for the popcount kernel and as the yardstick the matrix-core kernel has
+# to beat.  A SIMD issues one wave64 VALU instruction in `cycles`: measured on MI355X with
+# tab_amd/lib/valu_peak (profiles/valu_issue_rates.txt): 2 cycles for v_xor/v_and/v_bitop3
+# (128 lanes/clk/CU) and 4 cycles for v_bcnt_u32_b32 (64 lanes/clk/CU).  Per 32-bit word pair
+# (= 64 binary ops per lane) the popcount kernels issue
 #   BNN xor+bcnt = 6, TBN/BTN bitop3+bcnt = 6, TNN and+bcnt+bitop3+bcnt = 12 cycles.
 # peak = 256 CUs x 4 SIMDs x 2.4 GHz x 64 lanes x 64 binary ops / cycles.
 SIMD_HZ = 256 * 4 * 2.4e9
@@ -32,16 +37,35 @@ ISSUED_CYCLES_PER_PAIR = {0: 12, 1: 6, 2: 6, 3: 6}
 # (TAB_GEMM.cu:48-51,81-84,113-114,142): TNN 5, TBN 4, BTN 3, BNN 2 lane-ops per pair.
 REFERENCE_MIX_OPS = {0: 5, 1: 4, 2: 3, 3: 2}
 HBM_PEAK_GBS = 8000.0
+# HBM bytes moved by the ten conv launches of one headline step, from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE passes over `bench.py --profile` scaled by a 256 MiB copy
+# (profiles/quantize_conv_profile_sequence_traffic.txt).
+CONV_STEP_TRAFFIC_BYTES = 59132199
 
 
 def valu_peak_tops(type):
-    """Roofline of the instruction mix the kernel really issues, at the measured issue rates."""
+    """Roofline of the instruction mix the popcount kernel really issues, at the measured issue rates."""
     return SIMD_HZ * 64 * 64 / ISSUED_CYCLES_PER_PAIR[type] / 1e12
 
 
 def planning_peak_tops(type):
     """256 CU x 64 lanes x 2.4 GHz lane-ops/s over the reference's op mix."""
     return 256 * 64 * 2.4e9 * 64 / REFERENCE_MIX_OPS[type] / 1e12
+
+
+def layer_bytes(N, layer, wbits=1):
+    """Algorithmic HBM bytes of one Conv2d call: X read, QW read, Y written."""
+    H, W, C, KN, KH, KW, p1, p2, s1, s2 = layer
+    OH, OW = out_extent(H, p1, KH, s1), out_extent(W, p2, KW, s2)
+    return 4 * N * H * W * C + 8 * KN * KH * KW * ((C + 63) // 64) * wbits + 4 * N * OH * OW * KN
+
+
+def conv_kernel_bytes(N, layer, abits=1, wbits=1):
+    """Algorithmic HBM bytes of the conv kernel alone: packed activation and weights read, Y written."""
+    H, W, C, KN, KH, KW, p1, p2, s1, s2 = layer
+    OH, OW = out_extent(H, p1, KH, s1), out_extent(W, p2, KW, s2)
+    PC = (C + 63) // 64
+    return 8 * N * H * W * PC * abits + 8 * KN * KH * KW * PC * wbits + 4 * N * OH * OW * KN
 
 
 # (H, W, C, KN, KH, KW, pad1, pad2, stride1, stride2): ResNet-18 3x3 layers + stride-2 variants
@@ -190,7 +214,8 @@ def profile_sequence(torch, tab):
     """Launch sequence for counter collection: a plain 256 MiB device copy (the yardstick that
     FETCH_SIZE / WRITE_SIZE are scaled with), Quantize at the roofline shape for both bit
     widths, the conv kernel of every ResNet-18 N=16 layer, and the conv kernel of the large
-    sweep point for all four types.  Three repetitions each."""
+    sweep point for all four types: the default (matrix-core) kernel, then the popcount kernel on
+    the same tensors.  Three repetitions each."""
     src = torch.empty(256 * 1024 * 1024 // 4, dtype=torch.float32, device="cuda").normal_()
     dst = torch.empty_like(src)
     for _ in range(3):
@@ -210,8 +235,11 @@ def profile_sequence(torch, tab):
             L.conv_kernel_only()
     for type in range(4):
         L = Layer(tab, torch, type, 256, (28, 28, 512, 512, 3, 3, 1, 1, 1, 1), seed=7, on_device=True)
-        for _ in range(3):
-            L.conv_kernel_only()
+        for kernel in (tab.CONV_AUTO, tab.CONV_POPCOUNT):
+            tab.set_conv_kernel(kernel, -1)
+            for _ in range(3):
+                L.conv_kernel_only()
+        tab.set_conv_kernel(tab.CONV_AUTO, -1)
         del L
     torch.cuda.synchronize()
     print("profile sequence done")
@@ -285,22 +313,32 @@ def main():
         per_layer.append({"layer": layer_name(N, l.layer), "latency_us": round(call_ms * 1e3, 2),
                           "conv_kernel_us": round(k_ms * 1e3, 2), "quantize_kernel_us": round(q_ms * 1e3, 2),
                           "conv_kernel_tops": round(l.ops / k_ms / 1e9, 2),
-                          "frac_valu_peak": round(l.ops / k_ms / 1e9 / valu_peak_tops(3), 4)})
+                          "frac_mfma_peak": round(l.ops / k_ms / 1e9 / MFMA_FP4_PEAK_TOPS, 4),
+                          "hbm_floor_us": round(layer_bytes(N, l.layer) / HBM_PEAK_GBS / 1e3, 2)})
     achieved = conv_ops / conv_ms / 1e9  # TOP/s over the conv launches of one step
-    roofline = {"kernel": "conv_popcount<BNN>", "bound": "valu", "achieved": round(achieved, 2),
-                "peak": round(valu_peak_tops(3), 1), "unit": "TOP/s (effective binary ops)",
-                "frac": round(achieved / valu_peak_tops(3), 4), "traffic": None,
-                "frac_of_planning_peak": round(achieved / planning_peak_tops(3), 4),
-                "planning_peak": round(planning_peak_tops(3), 1),
-                "note": "peak = 1024 SIMDs x 2.4 GHz x 64 lanes x 64 binary ops / 6 issue cycles per 32-bit "
-                        "word pair (v_xor 2 + v_bcnt 4, measured issue rates); planning_peak = 256 CU x 64 "
-                        "lanes x 2.4 GHz / 2 lane-ops per pair; achieved = sum of layer ops / sum of average "
-                        "kernel durations (HIP events around graph replays of 20 launches per layer)"}
+    # the same launches with the popcount kernel, for the comparison the matrix-core kernel has to win
+    tab.set_conv_kernel(tab.CONV_POPCOUNT, -1)
+    popcount_ms = sum(graph_time_ms(torch, l.conv_kernel_only, 20) for l in layers)
+    tab.set_conv_kernel(tab.CONV_AUTO, -1)
+    roofline = {"kernel": "conv_mfma<BNN> (v_mfma_f32_32x32x64_f8f6f4, FP4 operands)", "bound": "mfma",
+                "achieved": round(achieved, 2), "peak": MFMA_FP4_PEAK_TOPS, "unit": "TFLOP/s",
+                "frac": round(achieved / MFMA_FP4_PEAK_TOPS, 4), "traffic": CONV_STEP_TRAFFIC_BYTES,
+                "algorithmic_bytes": sum(conv_kernel_bytes(N, l.layer) for l in layers),
+                "popcount_kernel_achieved": round(conv_ops / popcount_ms / 1e9, 2),
+                "valu_popcount_planning_peak": round(planning_peak_tops(3), 1),
+                "achieved_over_valu_planning_peak": round(achieved / planning_peak_tops(3), 4),
+                "note": "one effective binary op = one FP4 flop; peak = MI355X dense FP4 10.1 PFLOP/s; achieved = sum "
+                        "of layer ops / sum of average conv-kernel durations (HIP events around graph replays of 20 "
+                        "launches per layer) over the ten launches of one step, which at N=16 are launch- and "
+                        "latency-bound (see resnet18_bnn_N256 and sweep_N256_28x28x512_3x3 for kernels long enough "
+                        "to load the matrix cores); traffic (rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by a copy) and algorithmic_bytes (packed activation + weights + Y) are HBM bytes of the ten conv launches of one step; "
+                        "popcount_kernel_achieved is the VALU popcount kernel on the same launches, "
+                        "valu_popcount_planning_peak its roofline (256 CU x 64 lanes x 2.4 GHz / 2 lane-ops per pair)"}
 
     result = {
         "metric": "tab_conv2d_effective_binary_tops", "value": round(value, 3), "unit": "TOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u32 popcount -> i32 -> f32",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp4 (e2m1) x fp4 -> f32 accumulate, exact integers",
         "data": "synthetic",
         "config": {"workload": "BNN (type 3) ResNet-18 layer set, N=16: 4x 3x3 s1 + 3x 3x3 s2 + 3x 1x1 s2; "
                                "one step = Conv2d (quantize + conv) on all 10 layers, replayed as one HIP graph",
@@ -330,20 +368,28 @@ def main():
         result["quantize"] = {"shape": "256x56x56x256 fp32", "bound": "hbm", "peak_GBps": HBM_PEAK_GBS, **quant}
 
         # ---- the same ResNet-18 layer set at N=256 (kernels long enough not to be launch-bound)
-        rn_ops, rn_ms, rn_layers = 0, 0.0, []
+        rn_ops, rn_ms, rn_pop_ms, rn_layers = 0, 0.0, 0.0, []
         for i, l in enumerate(RESNET18_LAYERS):
             L = Layer(tab, torch, 3, 256, l, seed=i, on_device=True)
             k_ms = graph_time_ms(torch, L.conv_kernel_only, 5, replays=4)
             c_ms = graph_time_ms(torch, L.conv2d, 5, replays=4)
+            tab.set_conv_kernel(tab.CONV_POPCOUNT, -1)
+            p_ms = graph_time_ms(torch, L.conv_kernel_only, 5, replays=4)
+            tab.set_conv_kernel(tab.CONV_AUTO, -1)
             rn_ops += L.ops
             rn_ms += k_ms
+            rn_pop_ms += p_ms
+            hbm_us = layer_bytes(256, l) / HBM_PEAK_GBS / 1e3
             rn_layers.append({"layer": layer_name(256, l), "conv_kernel_us": round(k_ms * 1e3, 1),
                               "call_us": round(c_ms * 1e3, 1), "conv_kernel_tops": round(L.ops / k_ms / 1e9, 1),
-                              "frac_valu_peak": round(L.ops / k_ms / 1e9 / valu_peak_tops(3), 4)})
+                              "popcount_kernel_tops": round(L.ops / p_ms / 1e9, 1),
+                              "frac_mfma_peak": round(L.ops / k_ms / 1e9 / MFMA_FP4_PEAK_TOPS, 4),
+                              "hbm_floor_us": round(hbm_us, 1), "call_frac_of_hbm_floor": round(hbm_us / (c_ms * 1e3), 4)})
             del L
         result["resnet18_bnn_N256"] = {"conv_kernel_tops": round(rn_ops / rn_ms / 1e9, 1),
-                                       "frac_valu_peak": round(rn_ops / rn_ms / 1e9 / valu_peak_tops(3), 4),
-                                       "frac_of_planning_peak": round(rn_ops / rn_ms / 1e9 / planning_peak_tops(3), 4),
+                                       "popcount_kernel_tops": round(rn_ops / rn_pop_ms / 1e9, 1),
+                                       "frac_mfma_peak": round(rn_ops / rn_ms / 1e9 / MFMA_FP4_PEAK_TOPS, 4),
+                                       "over_valu_planning_peak": round(rn_ops / rn_ms / 1e9 / planning_peak_tops(3), 4),
                                        "layers": rn_layers}
 
         # ---- the largest sweep point, all four types (conv kernel only) --------------------
@@ -353,12 +399,16 @@ def main():
             L = Layer(tab, torch, type, 256, big, seed=7, relu=(type == 1), on_device=True)
             k_ms = graph_time_ms(torch, L.conv_kernel_only, 5, replays=4)
             call_ms = graph_time_ms(torch, L.conv2d, 3, replays=3)
+            tab.set_conv_kernel(tab.CONV_POPCOUNT, -1)
+            p_ms = graph_time_ms(torch, L.conv_kernel_only, 5, replays=4)
+            tab.set_conv_kernel(tab.CONV_AUTO, -1)
             sweep[TYPE_NAMES[type]] = {"conv_kernel_ms": round(k_ms, 3), "call_ms": round(call_ms, 3),
                                        "conv_kernel_tops": round(L.ops / k_ms / 1e9, 1),
-                                       "valu_peak_tops": round(valu_peak_tops(type), 1),
-                                       "frac_valu_peak": round(L.ops / k_ms / 1e9 / valu_peak_tops(type), 4),
-                                       "planning_peak_tops": round(planning_peak_tops(type), 1),
-                                       "frac_of_planning_peak": round(L.ops / k_ms / 1e9 / planning_peak_tops(type), 4)}
+                                       "frac_mfma_peak": round(L.ops / k_ms / 1e9 / MFMA_FP4_PEAK_TOPS, 4),
+                                       "popcount_kernel_tops": round(L.ops / p_ms / 1e9, 1),
+                                       "popcount_frac_valu_peak": round(L.ops / p_ms / 1e9 / valu_peak_tops(type), 4),
+                                       "valu_planning_peak_tops": round(planning_peak_tops(type), 1),
+                                       "over_valu_planning_peak": round(L.ops / k_ms / 1e9 / planning_peak_tops(type), 4)}
             del L
         result["sweep_N256_28x28x512_3x3"] = sweep
 

@@ -11,7 +11,7 @@ SOURCES = ["tab_capi.hip", "tab_conv.hip", "tab_conv_mfma_tnn.hip", "tab_conv_mf
 OBJ_DIR = os.path.join(LIB_DIR, "obj")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -packed-fp32-ops: keep the compiler from forming packed-FP32 VALU ops from float code.
-HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall",
+HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-result",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
@@ -27,6 +27,17 @@ def build_valu_peak():
     if proc.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + proc.stdout)
     return PEAK_BIN
+
+
+MFMA_PEAK_SRC = os.path.join(CSRC, "mfma_peak.hip")
+MFMA_PEAK_BIN = os.path.join(LIB_DIR, "mfma_peak")
+
+
+def build_mfma_peak():
+    """Standalone microbenchmark of the FP4 matrix-core rate with and without operand expansion."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    _hipcc([HIPCC] + HIP_FLAGS + ["-o", MFMA_PEAK_BIN, MFMA_PEAK_SRC])
+    return MFMA_PEAK_BIN
 
 
 def extension_path():
@@ -87,4 +98,5 @@ def build_library(verbose=False):
 if __name__ == "__main__":
     print(build_library(verbose=True))
     print(build_valu_peak())
+    print(build_mfma_peak())
     print(build_torch_extension(verbose=True))

@@ -1,0 +1,127 @@
+// Matrix-core microbenchmark for the conv roofline: (1) checks that the FP4 (E2M1) encodings the conv
+// kernel builds from packed bit planes multiply to exact integers in v_mfma_f32_32x32x64_f8f6f4 for
+// all four operand combinations, (2) measures the instruction's issue rate alone and with the
+// per-tile expansion work of each conv type in front of it (2x2 tiles per wave, as in the kernel's
+// 128x128 shape).  Register-resident: no memory traffic in the timed loops.
+#include <hip/hip_runtime.h>
+#include <cstdio>
+#include <cstdint>
+#include <cstdlib>
+#define CK(x) do { hipError_t e = (x); if (e != hipSuccess) { printf("err %s line %d\n", hipGetErrorString(e), __LINE__); return 1; } } while (0)
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+#define M0 0x11111111u
+#define M1 0x22222222u
+#define M2 0x44444444u
+#define M3 0x88888888u
+// E2M1 nibble: bit3 sign, bits 2:1 exponent, bit0 mantissa: 0001=0.5 0010=1 0100=2
+// A-side weights per nibble bit j: (0.5, 1, 2, 2); B-side: (2, 1, 0.5, 0.5)
+__device__ __forceinline__ v8i bin_a(uint32_t w)   // value (bit ? -1 : +1) * weight
+{
+    v8i r = {0, 0, 0, 0, 0, 0, 0, 0};
+    r[0] = (int)(((w << 3) & M3) | M0); r[1] = (int)(((w << 2) & M3) | M1); r[2] = (int)(((w << 1) & M3) | M2); r[3] = (int)((w & M3) | M2);
+    return r;
+}
+__device__ __forceinline__ v8i bin_b(uint32_t w)
+{
+    v8i r = {0, 0, 0, 0, 0, 0, 0, 0};
+    r[0] = (int)(((w << 3) & M3) | M2); r[1] = (int)(((w << 2) & M3) | M1); r[2] = (int)(((w << 1) & M3) | M0); r[3] = (int)((w & M3) | M0);
+    return r;
+}
+__device__ __forceinline__ v8i ter_a(uint32_t s, uint32_t z)   // nz * (sign ? -1 : +1) * weight
+{
+    v8i r = {0, 0, 0, 0, 0, 0, 0, 0};
+    r[0] = (int)((z & M0) | ((s << 3) & M3)); r[1] = (int)((z & M1) | ((s << 2) & M3));
+    r[2] = (int)((z & M2) | ((s << 1) & M3)); r[3] = (int)(((z >> 1) & M2) | (s & M3));
+    return r;
+}
+__device__ __forceinline__ v8i ter_b(uint32_t s, uint32_t z)
+{
+    v8i r = {0, 0, 0, 0, 0, 0, 0, 0};
+    r[0] = (int)(((z << 2) & M2) | ((s << 3) & M3)); r[1] = (int)((z & M1) | ((s << 2) & M3));
+    r[2] = (int)(((z >> 2) & M0) | ((s << 1) & M3)); r[3] = (int)(((z >> 3) & M0) | (s & M3));
+    return r;
+}
+__device__ __forceinline__ v16f mfma(v8i a, v8i b, v16f c) { return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 4, 4, 0, 0, 0, 0); }
+// A: [32 rows][2 dwords] planes s,z ; B: [32 cols][2 dwords]; mode bit0: A ternary, bit1: B ternary
+__global__ void k_check(const uint32_t *As, const uint32_t *Az, const uint32_t *Bs, const uint32_t *Bz, float *C, int mode)
+{
+    const int lane = threadIdx.x, r = lane & 31, kb = lane >> 5;
+    v8i a = (mode & 1) ? ter_a(As[r * 2 + kb], Az[r * 2 + kb]) : bin_a(As[r * 2 + kb]);
+    v8i b = (mode & 2) ? ter_b(Bs[r * 2 + kb], Bz[r * 2 + kb]) : bin_b(Bs[r * 2 + kb]);
+    v16f c = {0};
+    c = mfma(a, b, c);
+    for (int j = 0; j < 4; j++)
+        for (int i = 0; i < 4; i++) C[(8 * j + 4 * kb + i) * 32 + r] = c[4 * j + i];
+}
+// MODE 0: mfma only; 1: BNN expansions; 2: TNN expansions; 3: TBN
+template <int MODE>
+__global__ __launch_bounds__(256) void k_tput(float *out, int iters, uint32_t seed)
+{
+    v16f c[2][2];
+    for (int i = 0; i < 2; i++) for (int j = 0; j < 2; j++) for (int e = 0; e < 16; e++) c[i][j][e] = 0;
+    uint32_t w[8];
+    for (int i = 0; i < 8; i++) w[i] = seed * (threadIdx.x + 1) * (2 * i + 1);
+    v8i a[2], b[2];
+    for (int i = 0; i < 2; i++) { a[i] = bin_a(w[i]); b[i] = bin_b(w[2 + i]); }
+    for (int it = 0; it < iters; it++) {
+        if (MODE != 0) {
+            for (int i = 0; i < 2; i++) {
+                a[i] = (MODE == 1) ? bin_a(w[i]) : ter_a(w[i], w[4 + i]);
+                b[i] = (MODE == 2) ? ter_b(w[2 + i], w[6 + i]) : bin_b(w[2 + i]);
+            }
+            w[0] += 0x9e3779b9u; for (int i = 1; i < 8; i++) w[i] ^= w[i - 1];
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++) c[i][j] = mfma(a[i], b[j], c[i][j]);
+    }
+    float s = 0;
+    for (int i = 0; i < 2; i++) for (int j = 0; j < 2; j++) for (int e = 0; e < 16; e++) s += c[i][j][e];
+    if (s == 12345.678f) out[threadIdx.x] = s;
+}
+template <int MODE> int tput(const char *name, int bpc)
+{
+    float *out; CK(hipMalloc(&out, 4096));
+    const int iters = 4000, blocks = 256 * bpc;
+    hipEvent_t e0, e1; CK(hipEventCreate(&e0)); CK(hipEventCreate(&e1));
+    k_tput<MODE><<<blocks, 256>>>(out, 10, 3); CK(hipDeviceSynchronize());
+    CK(hipEventRecord(e0)); k_tput<MODE><<<blocks, 256>>>(out, iters, 3); CK(hipEventRecord(e1)); CK(hipEventSynchronize(e1));
+    float ms; CK(hipEventElapsedTime(&ms, e0, e1));
+    double macs = (double)blocks * 4 * iters * 4 * 32 * 32 * 64;
+    printf("%-28s blocks/CU=%d %.3f ms  %.0f binary-equivalent TOP/s; cycles per MFMA per SIMD @2.4GHz = %.1f\n", name, bpc, ms,
+           2 * macs / (ms * 1e-3) / 1e12, ms * 1e-3 * 2.4e9 / ((double)bpc * iters * 4));
+    CK(hipFree(out));
+    return 0;
+}
+static int val_t(uint32_t s, uint32_t z, int k) { return ((z >> k) & 1) ? (((s >> k) & 1) ? -1 : 1) : 0; }
+static int val_b(uint32_t w, int k) { return ((w >> k) & 1) ? -1 : 1; }
+int main()
+{
+    setvbuf(stdout, NULL, _IONBF, 0);
+    uint32_t h[4][64]; float hC[1024];
+    srand(7);
+    for (int p = 0; p < 4; p++) for (int i = 0; i < 64; i++) h[p][i] = ((uint32_t)rand() << 16) ^ (uint32_t)rand() ^ ((uint32_t)rand() << 31);
+    uint32_t *d[4]; float *dC;
+    for (int p = 0; p < 4; p++) { CK(hipMalloc(&d[p], 256)); CK(hipMemcpy(d[p], h[p], 256, hipMemcpyHostToDevice)); }
+    CK(hipMalloc(&dC, 4096));
+    for (int mode = 0; mode < 4; mode++) {
+        k_check<<<1, 64>>>(d[0], d[1], d[2], d[3], dC, mode); CK(hipDeviceSynchronize());
+        CK(hipMemcpy(hC, dC, 4096, hipMemcpyDeviceToHost));
+        int bad = 0;
+        for (int m = 0; m < 32; m++) for (int n = 0; n < 32; n++) {
+            int s = 0;
+            for (int k = 0; k < 64; k++) {
+                const int q = k >> 5, kk = k & 31;
+                const int av = (mode & 1) ? val_t(h[0][m * 2 + q], h[1][m * 2 + q], kk) : val_b(h[0][m * 2 + q], kk);
+                const int bv = (mode & 2) ? val_t(h[2][n * 2 + q], h[3][n * 2 + q], kk) : val_b(h[2][n * 2 + q], kk);
+                s += av * bv;
+            }
+            bad += hC[m * 32 + n] != (float)s;
+        }
+        printf("check A %s x B %s: %d mismatches of 1024 (C[0][0]=%g)\n", (mode & 1) ? "ternary" : "binary", (mode & 2) ? "ternary" : "binary", bad, hC[0]);
+    }
+    for (int bpc : {1, 2, 3}) { tput<0>("f4 mfma only", bpc); tput<1>("BNN expansions", bpc); tput<3>("TBN expansions", bpc); tput<2>("TNN expansions", bpc); }
+    return 0;
+}
