@@ -114,6 +114,21 @@ int tab_conv2d_packed(const int64_t *dev_QX, const int64_t *dev_QW, const int32_
                       int H, int W, int C, int KN, int KH, int KW, float *dev_Y, void *stream);
 
 /*
+ * tab_conv2d_packed with the output quantized and packed in the kernel's epilogue instead of written
+ * as fp32: dev_QY is what tab_quantize(Y, dev_out_ths, out_bitwidth, N, OH, OW, KN) would give for
+ * the Y of tab_conv2d_packed - Y's memory order (n, oh, ow, kn) read as the NHWC activation of the
+ * next layer (TAB_GEMM.cu:53,526 for the order; TAB_GEMM.cu:184-192, 231 for the compares) - bit
+ * for bit, without Y ever reaching memory.  It chains layers packed-in / packed-out; the
+ * reference has no counterpart (every TAB_Conv2d returns fp32 and the caller re-quantizes).
+ *   dev_out_ths fp32 [>=N]: threshold for the outputs of image n
+ *   dev_QY      int64 [N*OH*OW*ceil(KN/64)*out_bitwidth], every element is written
+ */
+int tab_conv2d_packed_out(const int64_t *dev_QX, const int64_t *dev_QW, const int32_t *dev_btn,
+                          int type, int padding1, int padding2, int stride1, int stride2, int N,
+                          int H, int W, int C, int KN, int KH, int KW, const float *dev_out_ths,
+                          int out_bitwidth, int64_t *dev_QY, void *stream);
+
+/*
  * Which kernel tab_conv2d / tab_conv2d_packed launch.  Both give bit-identical Y; the switch exists
  * for verification and tuning and has no counterpart in the reference (which has one GEMM kernel
  * per type, TAB_GEMM.cu:25-147).  Process-wide, not thread-safe against concurrent conv calls.

@@ -168,6 +168,37 @@ def Conv2dPacked(QX, QW, btn, type, padding1, padding2, stride1, stride2, N, H, 
     return Y
 
 
+def Conv2dPackedOut(QX, QW, btn, type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW,
+                    out_thresholds, out_bitwidth):
+    """Conv2dPacked whose output is quantized and packed in the kernel's epilogue: returns QY int64
+    (N, OH, OW, ceil(KN/64), out_bitwidth), equal bit for bit to
+    Quantize(Conv2dPacked(...), out_thresholds, out_bitwidth, N, OH, OW, KN)[0] - the conv output's
+    (n, oh, ow, kn) memory read as the next layer's NHWC activation - without the fp32 tensor ever
+    being written.  out_thresholds: fp32 [>=N], one threshold per image."""
+    for t, name in ((QX, "QX"), (QW, "QW"), (btn, "btn"), (out_thresholds, "out_thresholds")):
+        _check_input(t, name)
+    _check_dtype(QX, torch.int64, "QX")
+    _check_dtype(QW, torch.int64, "QW")
+    _check_dtype(btn, torch.int32, "btn")
+    _check_dtype(out_thresholds, torch.float32, "out_thresholds")
+    (type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW, out_bitwidth) = (
+        int(v) for v in (type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW, out_bitwidth))
+    OH, OW = _conv_checks(QW, btn, type, N, H, W, C, KN, KH, KW, padding1, padding2, stride1, stride2)
+    abits = 2 if type < 2 else 1
+    if QX.numel() != N * H * W * packed_channels(C) * abits:
+        raise RuntimeError(f"QX has {QX.numel()} words, type {type} expects N*H*W*PC*{abits}")
+    if out_thresholds.numel() < N:
+        raise RuntimeError(f"out_thresholds has {out_thresholds.numel()} elements, need N={N}")
+    if out_bitwidth not in (1, 2):
+        raise RuntimeError(f"out_bitwidth must be 1 or 2, got {out_bitwidth}")
+    with torch.cuda.device(QX.device):
+        QY = torch.empty((N, OH, OW, packed_channels(KN), out_bitwidth), dtype=torch.int64, device=QX.device)
+        _capi.check(_lib, _lib.tab_conv2d_packed_out(QX.data_ptr(), QW.data_ptr(), btn.data_ptr(), type,
+                                                     padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW,
+                                                     out_thresholds.data_ptr(), out_bitwidth, QY.data_ptr(), _stream()))
+    return QY
+
+
 CONV_AUTO, CONV_MATRIX, CONV_POPCOUNT = 0, 1, 2
 
 
@@ -181,6 +212,6 @@ def set_conv_kernel(kernel=CONV_AUTO, tile=-1):
 TAB_Quantize = Quantize
 TAB_Conv2d = Conv2d
 
-__all__ = ["Quantize", "Conv2d", "Conv2dPacked", "Threshold", "TAB_Quantize", "TAB_Conv2d", "TabError",
+__all__ = ["Quantize", "Conv2d", "Conv2dPacked", "Conv2dPackedOut", "Threshold", "TAB_Quantize", "TAB_Conv2d", "TabError",
            "packed_channels", "out_shape", "version", "TNN", "TBN", "BTN", "BNN", "set_conv_kernel",
            "CONV_AUTO", "CONV_MATRIX", "CONV_POPCOUNT"]

@@ -23,6 +23,7 @@ SIGNATURES = {
     "tab_conv2d_workspace_bytes": (_sz, [_int] * 5),
     "tab_conv2d": (_int, [_vp] * 4 + [_int] * 12 + [_vp, _vp, _sz, _vp]),
     "tab_conv2d_packed": (_int, [_vp] * 3 + [_int] * 12 + [_vp, _vp]),
+    "tab_conv2d_packed_out": (_int, [_vp] * 3 + [_int] * 12 + [_vp, _int, _vp, _vp]),
     "tab_set_conv_kernel": (_int, [_int, _int]),
 }
 

@@ -140,23 +140,33 @@ size_t tab_conv2d_workspace_bytes(int type, int N, int H, int W, int C)
     return (size_t)N * H * W * tab_packed_channels(C) * abits * sizeof(int64_t);
 }
 
-int tab_conv2d_packed(const int64_t *dev_QX, const int64_t *dev_QW, const int32_t *dev_btn,
-                      int type, int padding1, int padding2, int stride1, int stride2, int N,
-                      int H, int W, int C, int KN, int KH, int KW, float *dev_Y, void *stream)
+/* Shared body of the packed-activation entry points: Y as fp32 (dev_Y) or thresholded and packed (dev_QY). */
+static int conv_packed(const int64_t *dev_QX, const int64_t *dev_QW, const int32_t *dev_btn, int type, int padding1,
+                       int padding2, int stride1, int stride2, int N, int H, int W, int C, int KN, int KH, int KW,
+                       float *dev_Y, const float *dev_out_ths, int out_bitwidth, int64_t *dev_QY, void *stream)
 {
     ConvShape s;
     int rc = check_conv(type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW, &s);
     if (rc != TAB_OK) return rc;
-    if (!dev_QX || !dev_QW || !dev_Y) return fail(TAB_ERR_BAD_ARGUMENT, "null device pointer");
+    if (!dev_QX || !dev_QW || (!dev_Y && !dev_QY)) return fail(TAB_ERR_BAD_ARGUMENT, "null device pointer");
     if (type == TAB_BTN && !dev_btn) return fail(TAB_ERR_BAD_ARGUMENT, "btn is required for type 2 (BTN)");
     if (((uintptr_t)dev_QX % (8 * s.abits)) || ((uintptr_t)dev_QW % (8 * s.wbits)) || ((uintptr_t)dev_Y % 16))
         return fail(TAB_ERR_BAD_ARGUMENT, "QX/QW must be aligned to a whole packed element and Y to 16 bytes");
+    if (dev_QY) {
+        if (out_bitwidth != 1 && out_bitwidth != 2)
+            return fail(TAB_ERR_BAD_ARGUMENT, "out_bitwidth must be 1 or 2, got %d", out_bitwidth);
+        if (!dev_out_ths) return fail(TAB_ERR_BAD_ARGUMENT, "null device pointer");
+        if ((uintptr_t)dev_QY % (8 * out_bitwidth)) return fail(TAB_ERR_BAD_ARGUMENT, "QY must be aligned to a whole packed element");
+    }
 
     tab::ConvArgs a;
     a.qx = reinterpret_cast<const uint64_t *>(dev_QX);
     a.qw = reinterpret_cast<const uint64_t *>(dev_QW);
     a.btn = dev_btn;
     a.y = dev_Y;
+    a.qy = reinterpret_cast<uint32_t *>(dev_QY);
+    a.out_ths = dev_out_ths;
+    a.out_bits = out_bitwidth;
     a.N = N; a.H = H; a.W = W; a.PC = s.PC;
     a.KN = KN; a.KH = KH; a.KW = KW;
     a.p1 = padding1; a.p2 = padding2; a.s1 = stride1; a.s2 = stride2;
@@ -170,6 +180,25 @@ int tab_conv2d_packed(const int64_t *dev_QX, const int64_t *dev_QW, const int32_
     hipError_t e = tab::launch_conv(type, a, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return device_fail(e, "conv launch");
     return TAB_OK;
+}
+
+int tab_conv2d_packed(const int64_t *dev_QX, const int64_t *dev_QW, const int32_t *dev_btn,
+                      int type, int padding1, int padding2, int stride1, int stride2, int N,
+                      int H, int W, int C, int KN, int KH, int KW, float *dev_Y, void *stream)
+{
+    if (!dev_Y) return fail(TAB_ERR_BAD_ARGUMENT, "null device pointer");
+    return conv_packed(dev_QX, dev_QW, dev_btn, type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW,
+                       dev_Y, nullptr, 0, nullptr, stream);
+}
+
+int tab_conv2d_packed_out(const int64_t *dev_QX, const int64_t *dev_QW, const int32_t *dev_btn,
+                          int type, int padding1, int padding2, int stride1, int stride2, int N,
+                          int H, int W, int C, int KN, int KH, int KW, const float *dev_out_ths,
+                          int out_bitwidth, int64_t *dev_QY, void *stream)
+{
+    if (!dev_QY) return fail(TAB_ERR_BAD_ARGUMENT, "null device pointer");
+    return conv_packed(dev_QX, dev_QW, dev_btn, type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW,
+                       nullptr, dev_out_ths, out_bitwidth, dev_QY, stream);
 }
 
 int tab_conv2d(const float *dev_X, const int64_t *dev_QW, const float *dev_ths,

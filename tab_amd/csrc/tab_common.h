@@ -33,6 +33,10 @@ struct ConvArgs {
     const uint64_t *qw;  // packed weight     [KN][KH][KW][PC][BPL]
     const int32_t *btn;  // [KN] (BTN only)
     float *y;            // [M][KN]
+    // packed output instead of y (matrix-core kernel only): 32-bit halves of [M][ceil(KN/64)][out_bits]
+    uint32_t *qy;
+    const float *out_ths;  // [N] thresholds applied to the outputs of image n
+    int out_bits;          // 1 or 2
     int N, H, W, PC;
     int KN, KH, KW;
     int p1, p2, s1, s2;

@@ -353,12 +353,17 @@ int conv_mfma_shape(const ConvArgs &a)
     auto tiles = [&](int bm, int bn) { return (long)((a.M + bm - 1) / bm) * ((a.KN + bn - 1) / bn); };
     if (a.KN > 64 && tiles(128, 128) >= 1024) return 0;
     if (tiles(128, 64) >= 1024) return 1;
-    if (tiles(64, 64) >= 192) return 2;
+    if (tiles(64, 64) >= 192 || a.qy != nullptr) return 2;  // the packed epilogue needs tiles 64 filters wide
     return 3;
 }
 
 hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream)
 {
+    if (args.qy != nullptr) {  // packed output exists in the matrix-core kernel's 64-wide shapes only
+        if (!conv_mfma_exact(args)) return hipErrorInvalidValue;
+        const int shape = (g_force_tm == 9 && g_force_ng >= 0 && g_force_ng <= 2) ? g_force_ng : conv_mfma_shape(args);
+        return launch_conv_mfma(type, args, shape, stream);
+    }
     if (g_force_tm == 9) return launch_conv_mfma(type, args, g_force_ng < 0 ? conv_mfma_shape(args) : g_force_ng, stream);
     // default path: matrix cores; the popcount kernel takes over when K is too long for exact fp32
     // accumulation (and when a benchmark forces one of its tiles)

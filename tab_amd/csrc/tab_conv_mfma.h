@@ -192,6 +192,63 @@ __global__ __launch_bounds__(kConvThreads) void conv_mfma(const ConvArgs p)
         }
         return;
     }
+    if (p.qy != nullptr) {
+        // Packed output: Y is not written; each value is thresholded like the quantizer would
+        // threshold it as the next layer's NHWC activation (item = image, channel = filter;
+        // TAB_GEMM.cu:184-192, 231) and a wave ballot is 32 channels of two output pixels: lanes
+        // 0-31 hold row 8j+i, lanes 32-63 row 8j+4+i, so each half of the ballot is one 32-bit
+        // half of a packed word.  Tiles are multiples of 64 filters wide here, so every word that
+        // exists is written completely, tail bits as zeros.
+        const int pixels = p.OH * p.OW;
+        const int n_first = wave_m0 / pixels, rem0 = wave_m0 - n_first * pixels;  // uniform
+        const int out_words = (p.KN + 63) >> 6;
+        float bias[TN];
+        bool col_ok[TN];
+#pragma unroll
+        for (int nt = 0; nt < TN; nt++) {
+            const int col = wave_n0 + nt * 32 + r;
+            col_ok[nt] = col < p.KN;
+            bias[nt] = 0.f;
+            if (TYPE == 2) {
+                const int nonzero = b_nonzero[nt] + __shfl_xor(b_nonzero[nt], 32, 64);
+                bias[nt] = (float)((col_ok[nt] ? p.btn[col] : 0) - nonzero);
+            }
+            if (TYPE == 3) bias[nt] = (float)(p.num - 64 * p.nchunks * KCH);
+        }
+#pragma unroll
+        for (int mt = 0; mt < TM; mt++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int ro = mt * 32 + 8 * j + 4 * kb + i;
+                    const int m = wave_m0 + ro;
+                    const int past = rem0 + ro;  // pixels past the start of image n_first
+                    int n = n_first + (past >= pixels ? past / pixels : 0);
+                    n = n < p.N ? n : p.N - 1;  // rows past M are computed but not stored
+                    const float th = p.out_ths[n];
+#pragma unroll
+                    for (int nt = 0; nt < TN; nt++) {
+                        const float v = acc[mt][nt][4 * j + i] + bias[nt];
+                        const int col0 = wave_n0 + nt * 32;  // uniform
+                        if (col0 >= 64 * out_words) continue;
+                        const size_t word = (size_t)m * out_words + (col0 >> 6);
+                        const int half = (col0 >> 5) & 1;
+                        if (p.out_bits == 1) {
+                            const uint64_t b = __ballot(col_ok[nt] && v < th);
+                            if (r == 0 && m < p.M) p.qy[word * 2 + half] = kb ? (uint32_t)(b >> 32) : (uint32_t)b;
+                        } else {
+                            const bool pos = v > th, neg = !pos && v < -th;
+                            const uint64_t sg = __ballot(col_ok[nt] && neg), nz = __ballot(col_ok[nt] && (pos || neg));
+                            if (r == 0 && m < p.M) {
+                                p.qy[(word * 2 + 0) * 2 + half] = kb ? (uint32_t)(sg >> 32) : (uint32_t)sg;
+                                p.qy[(word * 2 + 1) * 2 + half] = kb ? (uint32_t)(nz >> 32) : (uint32_t)nz;
+                            }
+                        }
+                    }
+                }
+        return;
+    }
 #pragma unroll
     for (int nt = 0; nt < TN; nt++) {
         const int col = wave_n0 + nt * 32 + r;
