@@ -128,6 +128,12 @@ class Layer:
     def conv_kernel_only(self):
         return self.tab.Conv2dPacked(self.QX, self.QW, self.BTN, *self.args)
 
+    def conv_packed_out(self):
+        """Packed in, packed out (1-bit, threshold 0): what a chained binary layer runs."""
+        if not hasattr(self, "out_ths"):
+            self.out_ths = self.x_ths.new_zeros(self.N)
+        return self.tab.Conv2dPackedOut(self.QX, self.QW, self.BTN, *self.args, self.out_ths, 1)
+
     def quantize_only(self):
         _, p1, p2, s1, s2, N, H, W, C, KN, KH, KW = self.args
         return self.tab.Quantize(self.x, self.x_ths, self.abits, N, H, W, C)
@@ -368,7 +374,7 @@ def main():
         result["quantize"] = {"shape": "256x56x56x256 fp32", "bound": "hbm", "peak_GBps": HBM_PEAK_GBS, **quant}
 
         # ---- the same ResNet-18 layer set at N=256 (kernels long enough not to be launch-bound)
-        rn_ops, rn_ms, rn_pop_ms, rn_layers = 0, 0.0, 0.0, []
+        rn_ops, rn_ms, rn_pop_ms, rn_out_ms, rn_call_ms, rn_layers = 0, 0.0, 0.0, 0.0, 0.0, []
         for i, l in enumerate(RESNET18_LAYERS):
             L = Layer(tab, torch, 3, 256, l, seed=i, on_device=True)
             k_ms = graph_time_ms(torch, L.conv_kernel_only, 5, replays=4)
@@ -376,18 +382,27 @@ def main():
             tab.set_conv_kernel(tab.CONV_POPCOUNT, -1)
             p_ms = graph_time_ms(torch, L.conv_kernel_only, 5, replays=4)
             tab.set_conv_kernel(tab.CONV_AUTO, -1)
+            o_ms = graph_time_ms(torch, L.conv_packed_out, 5, replays=4)
             rn_ops += L.ops
             rn_ms += k_ms
             rn_pop_ms += p_ms
+            rn_out_ms += o_ms
+            rn_call_ms += c_ms
             hbm_us = layer_bytes(256, l) / HBM_PEAK_GBS / 1e3
             rn_layers.append({"layer": layer_name(256, l), "conv_kernel_us": round(k_ms * 1e3, 1),
                               "call_us": round(c_ms * 1e3, 1), "conv_kernel_tops": round(L.ops / k_ms / 1e9, 1),
                               "popcount_kernel_tops": round(L.ops / p_ms / 1e9, 1),
+                              "packed_out_us": round(o_ms * 1e3, 1), "packed_out_tops": round(L.ops / o_ms / 1e9, 1),
                               "frac_mfma_peak": round(L.ops / k_ms / 1e9 / MFMA_FP4_PEAK_TOPS, 4),
                               "hbm_floor_us": round(hbm_us, 1), "call_frac_of_hbm_floor": round(hbm_us / (c_ms * 1e3), 4)})
             del L
         result["resnet18_bnn_N256"] = {"conv_kernel_tops": round(rn_ops / rn_ms / 1e9, 1),
                                        "popcount_kernel_tops": round(rn_ops / rn_pop_ms / 1e9, 1),
+                                       "call_tops": round(rn_ops / rn_call_ms / 1e9, 1),
+                                       "packed_in_packed_out_tops": round(rn_ops / rn_out_ms / 1e9, 1),
+                                       "note": "conv_kernel = Conv2dPacked (packed in, fp32 out); call = Conv2d (fp32 in, fp32 out: "
+                                               "quantize + conv); packed_in_packed_out = Conv2dPackedOut (1-bit output packed in "
+                                               "the epilogue, what a chained binary layer runs)",
                                        "frac_mfma_peak": round(rn_ops / rn_ms / 1e9 / MFMA_FP4_PEAK_TOPS, 4),
                                        "over_valu_planning_peak": round(rn_ops / rn_ms / 1e9 / planning_peak_tops(3), 4),
                                        "layers": rn_layers}

@@ -202,6 +202,15 @@ __global__ __launch_bounds__(kConvThreads) void conv_mfma(const ConvArgs p)
         const int pixels = p.OH * p.OW;
         const int n_first = wave_m0 / pixels, rem0 = wave_m0 - n_first * pixels;  // uniform
         const int out_words = (p.KN + 63) >> 6;
+        // lane L (and L+32) looks up the threshold of row L of each 32-row tile and later stores
+        // that row's half-words
+        float th_row[TM];
+#pragma unroll
+        for (int mt = 0; mt < TM; mt++) {
+            int n = n_first + (rem0 + mt * 32 + r) / pixels;
+            n = n < p.N ? n : p.N - 1;  // rows past M are computed but not stored
+            th_row[mt] = p.out_ths[n];
+        }
         float bias[TN];
         bool col_ok[TN];
 #pragma unroll
@@ -216,37 +225,47 @@ __global__ __launch_bounds__(kConvThreads) void conv_mfma(const ConvArgs p)
             if (TYPE == 3) bias[nt] = (float)(p.num - 64 * p.nchunks * KCH);
         }
 #pragma unroll
-        for (int mt = 0; mt < TM; mt++)
+        for (int mt = 0; mt < TM; mt++) {
+            uint32_t sign_half[TN], nz_half[TN];  // of row r, meaningful in lanes 0-31
+#pragma unroll
+            for (int nt = 0; nt < TN; nt++) sign_half[nt] = nz_half[nt] = 0;
 #pragma unroll
             for (int j = 0; j < 4; j++)
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    const int ro = mt * 32 + 8 * j + 4 * kb + i;
-                    const int m = wave_m0 + ro;
-                    const int past = rem0 + ro;  // pixels past the start of image n_first
-                    int n = n_first + (past >= pixels ? past / pixels : 0);
-                    n = n < p.N ? n : p.N - 1;  // rows past M are computed but not stored
-                    const float th = p.out_ths[n];
+                    const int row_lo = 8 * j + i, row_hi = row_lo + 4;  // rows held by lanes 0-31 / 32-63
+                    const float th_lo = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(th_row[mt]), row_lo));
+                    const float th_hi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(th_row[mt]), row_hi));
+                    const float th = kb ? th_hi : th_lo;
 #pragma unroll
                     for (int nt = 0; nt < TN; nt++) {
                         const float v = acc[mt][nt][4 * j + i] + bias[nt];
-                        const int col0 = wave_n0 + nt * 32;  // uniform
-                        if (col0 >= 64 * out_words) continue;
-                        const size_t word = (size_t)m * out_words + (col0 >> 6);
-                        const int half = (col0 >> 5) & 1;
                         if (p.out_bits == 1) {
                             const uint64_t b = __ballot(col_ok[nt] && v < th);
-                            if (r == 0 && m < p.M) p.qy[word * 2 + half] = kb ? (uint32_t)(b >> 32) : (uint32_t)b;
+                            sign_half[nt] = r == row_lo ? (uint32_t)b : (r == row_hi ? (uint32_t)(b >> 32) : sign_half[nt]);
                         } else {
                             const bool pos = v > th, neg = !pos && v < -th;
                             const uint64_t sg = __ballot(col_ok[nt] && neg), nz = __ballot(col_ok[nt] && (pos || neg));
-                            if (r == 0 && m < p.M) {
-                                p.qy[(word * 2 + 0) * 2 + half] = kb ? (uint32_t)(sg >> 32) : (uint32_t)sg;
-                                p.qy[(word * 2 + 1) * 2 + half] = kb ? (uint32_t)(nz >> 32) : (uint32_t)nz;
-                            }
+                            sign_half[nt] = r == row_lo ? (uint32_t)sg : (r == row_hi ? (uint32_t)(sg >> 32) : sign_half[nt]);
+                            nz_half[nt] = r == row_lo ? (uint32_t)nz : (r == row_hi ? (uint32_t)(nz >> 32) : nz_half[nt]);
                         }
                     }
                 }
+            const int m = wave_m0 + mt * 32 + r;
+#pragma unroll
+            for (int nt = 0; nt < TN; nt++) {
+                const int col0 = wave_n0 + nt * 32;  // uniform
+                if (col0 >= 64 * out_words || lane >= 32 || m >= p.M) continue;
+                const size_t word = (size_t)m * out_words + (col0 >> 6);
+                const int half = (col0 >> 5) & 1;
+                if (p.out_bits == 1) {
+                    p.qy[word * 2 + half] = sign_half[nt];
+                } else {
+                    p.qy[(word * 2 + 0) * 2 + half] = sign_half[nt];
+                    p.qy[(word * 2 + 1) * 2 + half] = nz_half[nt];
+                }
+            }
+        }
         return;
     }
 #pragma unroll
