@@ -49,7 +49,7 @@ int check_conv(int type, int p1, int p2, int s1, int s2, int N, int H, int W, in
     s->wbits = (type == 0 || type == 2) ? 2 : 1;
     s->M = (long)N * s->OH * s->OW;
     s->G = (long)KH * KW * s->PC;
-    if (s->M > kMaxIndex || s->G >= 65536 || s->PC >= 65536 || KW >= 65536 ||
+    if (s->M > kMaxIndex - 512 || s->G >= 65536 || s->PC >= 65536 || KW >= 65536 ||
         (long)N * H * W > kMaxIndex || (long)H * W * s->PC * 2 > kMaxIndex)
         return fail(TAB_ERR_BAD_SHAPE, "problem too large for 32-bit row indices (M=%ld, K words=%ld)", s->M, s->G);
     // a workgroup addresses the images its (at most 256) output pixels touch with 32-bit byte offsets

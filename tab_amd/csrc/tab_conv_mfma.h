@@ -113,6 +113,27 @@ __global__ __launch_bounds__(kConvThreads) void conv_mfma(const ConvArgs p)
 #pragma unroll
     for (int nt = 0; nt < TN; nt++) b_nonzero[nt] = 0;
 
+    // Values the epilogue needs from memory are requested now, so their latency hides behind the
+    // main loop instead of stalling a workgroup that holds its registers and LDS: btn of this
+    // lane's filters (BTN) and, for packed output, the threshold of row r of each 32-row tile.
+    const int wave_m0 = m0 + wm * (32 * TM), wave_n0 = n0 + wn * (32 * TN);
+    int btn_col[TN];
+#pragma unroll
+    for (int nt = 0; nt < TN; nt++) {
+        const int col = wave_n0 + nt * 32 + r;
+        btn_col[nt] = (TYPE == 2 && col < p.KN) ? p.btn[col] : 0;
+    }
+    float th_row[TM];
+#pragma unroll
+    for (int mt = 0; mt < TM; mt++) {
+        th_row[mt] = 0.f;
+        if (p.qy != nullptr) {
+            int n = (wave_m0 + mt * 32 + r) / (p.OH * p.OW);
+            n = n < p.N ? n : p.N - 1;  // rows past M are computed but not stored
+            th_row[mt] = p.out_ths[n];
+        }
+    }
+
     st.fetch(p, 0);
     st.stage(lds);
     __syncthreads();
@@ -163,7 +184,6 @@ __global__ __launch_bounds__(kConvThreads) void conv_mfma(const ConvArgs p)
     }
 
     // ---- epilogue: accumulator element 4*j + i of lane (kb, r) is C[8*j + 4*kb + i][r] -------
-    const int wave_m0 = m0 + wm * (32 * TM), wave_n0 = n0 + wn * (32 * TN);
     const bool whole = wave_m0 + 32 * TM <= p.M && wave_n0 + 32 * TN <= p.KN;  // wave-uniform
     if (KS > 1) {
         // the KS waves hold partial sums of the same tile: exchange them through LDS; wave ks
@@ -183,7 +203,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_mfma(const ConvArgs p)
         const int col = wave_n0 + r;
         const bool col_ok = col < p.KN;
         float bias = 0.f;
-        if (TYPE == 2) bias = (float)(col_ok ? p.btn[col] : 0) - (sum[4] + __shfl_xor(sum[4], 32, 64));
+        if (TYPE == 2) bias = (float)btn_col[0] - (sum[4] + __shfl_xor(sum[4], 32, 64));
         if (TYPE == 3) bias = (float)(p.num - 64 * p.nchunks * KCH);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -199,18 +219,9 @@ __global__ __launch_bounds__(kConvThreads) void conv_mfma(const ConvArgs p)
         // 0-31 hold row 8j+i, lanes 32-63 row 8j+4+i, so each half of the ballot is one 32-bit
         // half of a packed word.  Tiles are multiples of 64 filters wide here, so every word that
         // exists is written completely, tail bits as zeros.
-        const int pixels = p.OH * p.OW;
-        const int n_first = wave_m0 / pixels, rem0 = wave_m0 - n_first * pixels;  // uniform
         const int out_words = (p.KN + 63) >> 6;
-        // lane L (and L+32) looks up the threshold of row L of each 32-row tile and later stores
+        // lane L (and L+32) holds the threshold of row L of each 32-row tile (th_row) and stores
         // that row's half-words
-        float th_row[TM];
-#pragma unroll
-        for (int mt = 0; mt < TM; mt++) {
-            int n = n_first + (rem0 + mt * 32 + r) / pixels;
-            n = n < p.N ? n : p.N - 1;  // rows past M are computed but not stored
-            th_row[mt] = p.out_ths[n];
-        }
         float bias[TN];
         bool col_ok[TN];
 #pragma unroll
@@ -220,7 +231,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_mfma(const ConvArgs p)
             bias[nt] = 0.f;
             if (TYPE == 2) {
                 const int nonzero = b_nonzero[nt] + __shfl_xor(b_nonzero[nt], 32, 64);
-                bias[nt] = (float)((col_ok[nt] ? p.btn[col] : 0) - nonzero);
+                bias[nt] = (float)(btn_col[nt] - nonzero);
             }
             if (TYPE == 3) bias[nt] = (float)(p.num - 64 * p.nchunks * KCH);
         }
@@ -275,7 +286,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_mfma(const ConvArgs p)
         float bias = 0.f;
         if (TYPE == 2) {
             const int nonzero = b_nonzero[nt] + __shfl_xor(b_nonzero[nt], 32, 64);
-            bias = (float)((col_ok ? p.btn[col] : 0) - nonzero);
+            bias = (float)(btn_col[nt] - nonzero);
         }
         if (TYPE == 3) bias = (float)(p.num - 64 * p.nchunks * KCH);
         float *out = p.y + (size_t)(wave_m0 + 4 * kb) * p.KN + col;
