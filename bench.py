@@ -427,6 +427,37 @@ def main():
             del L
         result["sweep_N256_28x28x512_3x3"] = sweep
 
+        # ---- more points of the large-batch sweep (BASELINE configs[4]): conv kernel TOP/s ----
+        # (C=KN, kernel, stride, pad1, pad2) at 28x28; asymmetric padding as the config asks
+        points = [(256, 3, 1, 1, 0), (512, 3, 2, 1, 0), (512, 1, 1, 0, 0), (256, 1, 2, 1, 0)]
+        more = {}
+        for n_batch in (64, 256):
+            for C, k, st, p1, p2 in points:
+                lay = (28, 28, C, C, k, k, p1, p2, st, st)
+                row = {}
+                for type in range(4):
+                    L = Layer(tab, torch, type, n_batch, lay, seed=3, on_device=True)
+                    row[TYPE_NAMES[type]] = round(L.ops / graph_time_ms(torch, L.conv_kernel_only, 5, replays=3) / 1e9, 1)
+                    del L
+                more[layer_name(n_batch, lay)] = row
+        result["sweep_more_conv_kernel_tops"] = more
+
+        # ---- TNN VGG-16-style stack at N=32 (BASELINE configs[3]) ---------------------------
+        vgg, vgg_ops, vgg_ms, vgg_call_ms = [], 0, 0.0, 0.0
+        for i, (hw, c) in enumerate([(224, 64), (112, 128), (56, 256), (28, 512), (14, 512)]):
+            lay = (hw, hw, c, c, 3, 3, 1, 1, 1, 1)
+            L = Layer(tab, torch, 0, 32, lay, seed=20 + i, on_device=True)
+            k_ms = graph_time_ms(torch, L.conv_kernel_only, 3, replays=3)
+            c_ms = graph_time_ms(torch, L.conv2d, 3, replays=3)
+            vgg_ops += L.ops
+            vgg_ms += k_ms
+            vgg_call_ms += c_ms
+            vgg.append({"layer": layer_name(32, lay), "conv_kernel_us": round(k_ms * 1e3, 1), "call_us": round(c_ms * 1e3, 1),
+                        "conv_kernel_tops": round(L.ops / k_ms / 1e9, 1)})
+            del L
+        result["vgg16_tnn_N32"] = {"conv_kernel_tops": round(vgg_ops / vgg_ms / 1e9, 1),
+                                   "call_tops": round(vgg_ops / vgg_call_ms / 1e9, 1), "layers": vgg}
+
         # ---- CPU baseline: the oracle on the same layer set, same tensors --------------------
         import oracle
 

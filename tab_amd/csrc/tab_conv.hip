@@ -345,14 +345,16 @@ hipError_t launch_conv_mfma(int type, const ConvArgs &args, int shape, hipStream
     }
 }
 
-// Workgroup tile of the matrix-core kernel, from measurements over the ResNet-18 and sweep layers at
-// N = 16 and N = 256: the largest tile that still gives the chip about four workgroups per CU; below
-// roughly 200 workgroups of 64x64 the launch is latency-bound and the k-split 32x32 shape wins.
+// Workgroup tile of the matrix-core kernel, from measurements over the ResNet-18, VGG and sweep layers at
+// N = 8 .. 256: the 128-row tiles win as soon as there is about one of them per CU (the 128x128 one
+// with short K they need about four per CU); below roughly 200 workgroups of 64x64 the launch is
+// latency-bound and the k-split 32x32 shape wins.
 int conv_mfma_shape(const ConvArgs &a)
 {
     auto tiles = [&](int bm, int bn) { return (long)((a.M + bm - 1) / bm) * ((a.KN + bn - 1) / bn); };
-    if (a.KN > 64 && tiles(128, 128) >= 1024) return 0;
-    if (tiles(128, 64) >= 1024) return 1;
+    const long enough = a.G >= 36 ? 300 : 1024;  // short K: the per-tile prologue and epilogue weigh more
+    if (a.KN > 64 && a.G >= 18 && tiles(128, 128) >= enough) return 0;
+    if (tiles(128, 64) >= enough) return 1;
     if (tiles(64, 64) >= 192 || a.qy != nullptr) return 2;  // the packed epilogue needs tiles 64 filters wide
     return 3;
 }
