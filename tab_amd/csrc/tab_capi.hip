@@ -213,6 +213,17 @@ int tab_conv2d(const float *dev_X, const int64_t *dev_QW, const float *dev_ths,
     const size_t need = tab_conv2d_workspace_bytes(type, N, H, W, C);
     if (!workspace || workspace_bytes < need || ((uintptr_t)workspace % 16))
         return fail(TAB_ERR_WORKSPACE, "workspace must be 16-byte aligned and hold %zu bytes (got %zu)", need, workspace_bytes);
+    // A 1x1 convolution with stride and no padding reads one pixel in stride1*stride2: quantize only
+    // those, into a compact activation, and convolve it with stride 1 (same outputs, a fraction of
+    // the reads of X).
+    if (KH == 1 && KW == 1 && padding1 == 0 && padding2 == 0 && (stride1 > 1 || stride2 > 1) && N * (long)s.OH < 65536 &&
+        tab::quantize_strided_supported(dev_X, H, W, C, s.OH, s.OW)) {
+        hipError_t e = tab::launch_quantize_strided(dev_X, dev_ths, s.abits, N, H, W, C, s.OH, s.OW, stride1, stride2,
+                                                    reinterpret_cast<uint64_t *>(workspace), static_cast<hipStream_t>(stream));
+        if (e != hipSuccess) return device_fail(e, "quantize launch");
+        return tab_conv2d_packed(reinterpret_cast<const int64_t *>(workspace), dev_QW, dev_btn, type, 0, 0, 1, 1, N, s.OH,
+                                 s.OW, C, KN, 1, 1, dev_Y, stream);
+    }
     // stage 1: quantize + pack the activation (TAB_GEMM.cu:419-426); no btn for activations
     hipError_t e = tab::launch_quantize(dev_X, dev_ths, s.abits, (long)H * W, N, C,
                                         reinterpret_cast<uint64_t *>(workspace), nullptr,

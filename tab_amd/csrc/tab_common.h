@@ -65,6 +65,12 @@ hipError_t launch_conv_mfma_bnn(const ConvArgs &args, int shape, hipStream_t str
 hipError_t launch_quantize(const float *x, const float *ths, int bitwidth, long pixels_per_item,
                            long items, int C, uint64_t *qx, int32_t *btn, hipStream_t stream);
 
+// Quantize only the pixels (oh*s1, ow*s2) of every image into a compact [N][OH][OW][PC] activation
+// (what a 1x1 convolution with stride and no padding reads).
+bool quantize_strided_supported(const float *x, int H, int W, int C, int OH, int OW);
+hipError_t launch_quantize_strided(const float *x, const float *ths, int bitwidth, int N, int H, int W, int C, int OH,
+                                   int OW, int s1, int s2, uint64_t *qx, hipStream_t stream);
+
 // ths[n] = scale * mean|x[n]| over per_item elements; `partial` holds items * threshold_splits()
 // floats of scratch.
 int threshold_splits(long items, long per_item);

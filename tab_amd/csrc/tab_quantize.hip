@@ -119,6 +119,52 @@ __global__ __launch_bounds__(kThreads) void quantize_rows64(const floatx4 *__res
     }
 }
 
+// The same row quantizer for a 1x1 convolution with stride and no padding, which reads only the
+// pixels (oh*s1, ow*s2): one wave per 32 consecutive words of one output line (n, oh); the packed
+// result is the compact [N][OH][OW][PC] activation, i.e. what the conv reads with stride 1.
+// grid = (ceil(OW*PC / 32), N*OH), one wave per workgroup; OW*PC < 65536 (fastdiv range).
+template <int BITS>
+__global__ __launch_bounds__(64) void quantize_rows64_strided(const floatx4 *__restrict__ x, const float *__restrict__ ths,
+                                                              uint32_t *__restrict__ q, int H, int W, int PC, int OH,
+                                                              int OW, int s1, int s2, FastDiv div_pc)
+{
+    const int lane = threadIdx.x;
+    const int sub = lane >> 4, l = lane & 15;
+    const int n = blockIdx.y / OH, oh = blockIdx.y - n * OH;  // uniform
+    const int line_words = OW * PC;
+    const long in_line = ((long)n * H + (long)oh * s1) * W;   // first input pixel of the line
+    const long out_line = (long)blockIdx.y * line_words;
+    const int j0 = blockIdx.x * kRowsPerWave;
+    const float t = ths[n];
+
+    floatx4 v[kLoadsPerLane];
+#pragma unroll
+    for (int u = 0; u < kLoadsPerLane; u++) {
+        const int j = j0 + u * 4 + sub;
+        const int ow = (int)fastdiv((uint32_t)j, div_pc), pc = j - ow * PC;
+        const long r = (in_line + (long)ow * s2) * PC + pc;
+        v[u] = (j < line_words) ? __builtin_nontemporal_load(&x[r * 16 + l]) : floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int u = 0; u < kLoadsPerLane; u++) {
+        const int j = j0 + u * 4 + sub;
+        const long r = out_line + j;
+        uint32_t sign, nz;
+        compare4<BITS>(v[u], t, sign, nz);
+        const int shift = 4 * (l & 7);
+        const uint32_t sign_half = or_reduce8(sign << shift);
+        const uint32_t sign_other = rotate_row8(sign_half);
+        if (BITS == 2) {
+            const uint32_t nz_half = or_reduce8(nz << shift);
+            const uint32_t nz_other = rotate_row8(nz_half);
+            if (j < line_words && l == 0)
+                *reinterpret_cast<uintx4 *>(q + r * 4) = uintx4{sign_half, sign_other, nz_half, nz_other};
+        } else {
+            if (j < line_words && l == 0) *reinterpret_cast<uintx2 *>(q + r * 2) = uintx2{sign_half, sign_other};
+        }
+    }
+}
+
 // General path (any C, any alignment): one wave per (pixel, word); lane i tests channel
 // word*64 + i and the two wave-wide ballots are the packed words, LSB first
 // (onebit[i] = 1 << i, TAB_GEMM.cu:252-258).  Unused high bits of a tail word stay 0
@@ -308,6 +354,26 @@ hipError_t launch_quantize(const float *x, const float *ths, int bitwidth, long 
         btn_popcount<<<dim3((unsigned)(items * splits)), dim3(kThreads), 0, stream>>>(
             reinterpret_cast<const ulonglong2 *>(qx), btn, words_per_item, splits);
     }
+    return hipGetLastError();
+}
+
+bool quantize_strided_supported(const float *x, int H, int W, int C, int OH, int OW)
+{
+    const long PC = C / kWordBits;
+    return C % kWordBits == 0 && (uintptr_t)x % 16 == 0 && OW * PC < 65536 && PC < 65536;
+}
+
+hipError_t launch_quantize_strided(const float *x, const float *ths, int bitwidth, int N, int H, int W, int C, int OH,
+                                   int OW, int s1, int s2, uint64_t *qx, hipStream_t stream)
+{
+    const int PC = C / kWordBits;
+    const dim3 grid((unsigned)((OW * PC + kRowsPerWave - 1) / kRowsPerWave), (unsigned)(N * OH)), block(64);
+    const floatx4 *x4 = reinterpret_cast<const floatx4 *>(x);
+    uint32_t *q32 = reinterpret_cast<uint32_t *>(qx);
+    if (bitwidth == 2)
+        quantize_rows64_strided<2><<<grid, block, 0, stream>>>(x4, ths, q32, H, W, PC, OH, OW, s1, s2, make_fastdiv(PC));
+    else
+        quantize_rows64_strided<1><<<grid, block, 0, stream>>>(x4, ths, q32, H, W, PC, OH, OW, s1, s2, make_fastdiv(PC));
     return hipGetLastError();
 }
 

@@ -48,6 +48,8 @@ EDGE_CASES = [
     (2, 12, 12, 192, 130, 3, 3, 1, 1, 1, 1),  # KN not a multiple of the 64/128 tile
     (1, 10, 10, 64, 66, 5, 5, 2, 2, 1, 1),    # 5x5 kernel
     (5, 4, 4, 1024, 12, 3, 3, 1, 1, 1, 1),    # long K (144 words)
+    (3, 9, 11, 192, 20, 1, 1, 0, 0, 2, 3),    # 1x1, no padding, strides (2, 3): only the pixels read are quantized
+    (2, 7, 8, 64, 70, 1, 1, 0, 0, 1, 2),      # 1x1, stride on W only
 ]
 
 
