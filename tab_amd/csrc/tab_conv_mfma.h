@@ -329,11 +329,15 @@ hipError_t launch_mfma_tile(ConvArgs a, hipStream_t stream)
     return hipGetLastError();
 }
 
-template <int TYPE, int WM, int WN, int TM, int TN>
+// LONG: the launch is small enough to be latency-bound, so prefer few long chunks (fewer serial
+// fetch round trips) over a small LDS footprint.
+template <int TYPE, int WM, int WN, int TM, int TN, bool LONG = false>
 hipError_t launch_mfma_shape(const ConvArgs &a, hipStream_t stream)
 {
     // chunks that stay inside one tap take the piece stager
+    if (LONG && a.PC % 8 == 0) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 8, true>(a, stream);
     if (a.PC % 4 == 0) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 4, true>(a, stream);
+    if (LONG && a.G % 9 == 0) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 9, false>(a, stream);
     if (a.PC % 2 == 0) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 2, true>(a, stream);
     switch (mfma_chunk_words(a.G)) {
     case 1: return launch_mfma_tile<TYPE, WM, WN, TM, TN, 1, false>(a, stream);
@@ -351,9 +355,11 @@ hipError_t launch_mfma_type(const ConvArgs &a, int shape, hipStream_t stream)
     switch (shape) {
     case 0: return launch_mfma_shape<TYPE, 2, 2, 2, 2>(a, stream);
     case 1: return launch_mfma_shape<TYPE, 4, 1, 1, 2>(a, stream);
-    case 2: return launch_mfma_shape<TYPE, 2, 2, 1, 1>(a, stream);
+    case 2: return launch_mfma_shape<TYPE, 2, 2, 1, 1, true>(a, stream);
     case 3:
+        if (a.PC % 8 == 0) return launch_mfma_tile<TYPE, 1, 1, 1, 1, 8, true, 4>(a, stream);
         if (a.PC % 4 == 0) return launch_mfma_tile<TYPE, 1, 1, 1, 1, 4, true, 4>(a, stream);
+        if (a.G > 4) return launch_mfma_tile<TYPE, 1, 1, 1, 1, 12, false, 4>(a, stream);
         return launch_mfma_tile<TYPE, 1, 1, 1, 1, 4, false, 4>(a, stream);
     default: return hipErrorInvalidValue;
     }
