@@ -75,8 +75,10 @@ __device__ __forceinline__ i32x8 expand_ternary(uint32_t s, uint32_t z)
     return r;
 }
 
+// waves_per_eu(4): at most 128 registers, i.e. four workgroups per CU; the 128x128 shape otherwise takes
+// 136-152 (64 of them accumulators) and runs three, measured 3-7 % slower.
 template <int TYPE, int WM, int WN, int TM, int TN, int KCH, bool INTAP, int KS = 1>
-__global__ __launch_bounds__(kConvThreads) void conv_mfma(const ConvArgs p)
+__global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(4))) void conv_mfma(const ConvArgs p)
 {
     static_assert(WM * WN * KS * 64 == kConvThreads, "four waves");
     static_assert(KCH % KS == 0 && (KS == 1 || (TM == 1 && TN == 1)), "k-split waves share one 32x32 tile");
