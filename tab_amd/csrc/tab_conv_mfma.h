@@ -147,7 +147,7 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(4)
 
         // Every chunk is exactly KCH words: the stager zero-fills words past the end of K, which add
         // nothing for a ternary operand and +64 per word for binary x binary (the BNN bias below
-        // counts them).  LDS reads run one word ahead of the matrix cores.
+        // counts them).
         const uint32_t *la = lds + (chunk & 1) * (A_DWORDS + B_DWORDS) + a_off, *lb = la - a_off + A_DWORDS + b_off;
         uint32_t a_w[WPW][APL][TM], b_w[WPW][BPL][TN];
         auto read_word = [&](int w) {
@@ -161,10 +161,19 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(4)
 #pragma unroll
                 for (int nt = 0; nt < TN; nt++) b_w[w][pl][nt] = lb[(pl * Q + q) * B_STRIDE + nt * 32];
         };
-        read_word(0);
+        // LDS reads run ahead of the matrix cores: the whole chunk up front when that is few registers
+        // (one-plane operands; measured +3 % on BNN, a loss for the two-plane types), else one word ahead
+        constexpr bool ALL_AHEAD = (APL * TM + BPL * TN) * WPW <= 16;
+        if (ALL_AHEAD) {
+#pragma unroll
+            for (int w = 0; w < WPW; w++) read_word(w);
+            __builtin_amdgcn_sched_barrier(0);
+        } else {
+            read_word(0);
+        }
 #pragma unroll
         for (int w = 0; w < WPW; w++) {
-            if (w + 1 < WPW) read_word(w + 1);
+            if (!ALL_AHEAD && w + 1 < WPW) read_word(w + 1);
             i32x8 af[TM], bf[TN];
 #pragma unroll
             for (int mt = 0; mt < TM; mt++)
@@ -337,9 +346,11 @@ template <int TYPE, int WM, int WN, int TM, int TN, bool LONG = false>
 hipError_t launch_mfma_shape(const ConvArgs &a, hipStream_t stream)
 {
     // chunks that stay inside one tap take the piece stager
-    if (LONG && a.PC % 8 == 0) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 8, true>(a, stream);
+    if constexpr (LONG)
+        if (a.PC % 8 == 0) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 8, true>(a, stream);
     if (a.PC % 4 == 0) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 4, true>(a, stream);
-    if (LONG && a.G % 9 == 0) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 9, false>(a, stream);
+    if constexpr (LONG)
+        if (a.G % 9 == 0) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 9, false>(a, stream);
     if (a.PC % 2 == 0) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 2, true>(a, stream);
     switch (mfma_chunk_words(a.G)) {
     case 1: return launch_mfma_tile<TYPE, WM, WN, TM, TN, 1, false>(a, stream);
