@@ -34,43 +34,49 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr uint32_t kBit0 = 0x11111111u, kBit1 = 0x22222222u, kBit2 = 0x44444444u, kBit3 = 0x88888888u;
 
-// (a & m) | c in one instruction.  This ISA takes no literal in a three-operand VALU instruction and
-// only one scalar register, so the mask rides in an SGPR and the other two operands in VGPRs; left
-// to itself the compiler emits a separate v_and and v_or with two literals.
-__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t m, uint32_t c)
-{
-    uint32_t r;
-    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(m), "v"(c));
-    return r;
-}
+// The constants of the expansion, made opaque to the optimiser and pinned to register classes:
+// this ISA takes no literal in a three-operand VALU instruction and only one scalar register, so
+// (x & sign_bits) | pattern becomes a single v_and_or_b32 only when the mask sits in an SGPR and the
+// pattern in a VGPR; with literals the compiler emits a v_and and a v_or.  (An inline-asm
+// v_and_or_b32 is not an option: the compiler's hazard recogniser does not see registers written by
+// inline asm and may then leave too few wait states before the MFMA that reads them.)
+struct ExpandConsts {
+    uint32_t sign_bits;          // kBit3, SGPR
+    uint32_t half, one, two;     // the E2M1 patterns of 0.5, 1, 2 in every nibble, VGPRs
+    __device__ __forceinline__ ExpandConsts() : sign_bits(kBit3), half(kBit0), one(kBit1), two(kBit2)
+    {
+        asm volatile("" : "+s"(sign_bits));
+        asm volatile("" : "+v"(half), "+v"(one), "+v"(two));
+    }
+};
 
 // SIDE 0 = activation (weights 0.5, 1, 2, 2), SIDE 1 = weight operand (2, 1, 0.5, 0.5)
 template <int SIDE>
-__device__ __forceinline__ i32x8 expand_binary(uint32_t w)
+__device__ __forceinline__ i32x8 expand_binary(uint32_t w, const ExpandConsts &c)
 {
-    constexpr uint32_t m0 = SIDE ? kBit2 : kBit0, m2 = SIDE ? kBit0 : kBit2;
+    const uint32_t m0 = SIDE ? c.two : c.half, m2 = SIDE ? c.half : c.two;
     i32x8 r = {0, 0, 0, 0, 0, 0, 0, 0};
-    r[0] = (int)and_or(w << 3, kBit3, m0);
-    r[1] = (int)and_or(w << 2, kBit3, kBit1);
-    r[2] = (int)and_or(w << 1, kBit3, m2);
-    r[3] = (int)and_or(w, kBit3, m2);
+    r[0] = (int)(((w << 3) & c.sign_bits) | m0);
+    r[1] = (int)(((w << 2) & c.sign_bits) | c.one);
+    r[2] = (int)(((w << 1) & c.sign_bits) | m2);
+    r[3] = (int)((w & c.sign_bits) | m2);
     return r;
 }
 
 template <int SIDE>
-__device__ __forceinline__ i32x8 expand_ternary(uint32_t s, uint32_t z)
+__device__ __forceinline__ i32x8 expand_ternary(uint32_t s, uint32_t z, const ExpandConsts &c)
 {
     i32x8 r = {0, 0, 0, 0, 0, 0, 0, 0};
     if (SIDE == 0) {
-        r[0] = (int)and_or(s << 3, kBit3, z & kBit0);
-        r[1] = (int)and_or(s << 2, kBit3, z & kBit1);
-        r[2] = (int)and_or(s << 1, kBit3, z & kBit2);
-        r[3] = (int)and_or(s, kBit3, (z >> 1) & kBit2);
+        r[0] = (int)(((s << 3) & c.sign_bits) | (z & kBit0));
+        r[1] = (int)(((s << 2) & c.sign_bits) | (z & kBit1));
+        r[2] = (int)(((s << 1) & c.sign_bits) | (z & kBit2));
+        r[3] = (int)((s & c.sign_bits) | ((z >> 1) & kBit2));
     } else {
-        r[0] = (int)and_or(s << 3, kBit3, (z << 2) & kBit2);
-        r[1] = (int)and_or(s << 2, kBit3, z & kBit1);
-        r[2] = (int)and_or(s << 1, kBit3, (z >> 2) & kBit0);
-        r[3] = (int)and_or(s, kBit3, (z >> 3) & kBit0);
+        r[0] = (int)(((s << 3) & c.sign_bits) | ((z << 2) & kBit2));
+        r[1] = (int)(((s << 2) & c.sign_bits) | (z & kBit1));
+        r[2] = (int)(((s << 1) & c.sign_bits) | ((z >> 2) & kBit0));
+        r[3] = (int)((s & c.sign_bits) | ((z >> 3) & kBit0));
     }
     return r;
 }
@@ -103,6 +109,7 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(4)
 
     Stager st;
     st.init(p, tid, m0, n0);
+    const ExpandConsts consts;
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -115,26 +122,7 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(4)
 #pragma unroll
     for (int nt = 0; nt < TN; nt++) b_nonzero[nt] = 0;
 
-    // Values the epilogue needs from memory are requested now, so their latency hides behind the
-    // main loop instead of stalling a workgroup that holds its registers and LDS: btn of this
-    // lane's filters (BTN) and, for packed output, the threshold of row r of each 32-row tile.
     const int wave_m0 = m0 + wm * (32 * TM), wave_n0 = n0 + wn * (32 * TN);
-    int btn_col[TN];
-#pragma unroll
-    for (int nt = 0; nt < TN; nt++) {
-        const int col = wave_n0 + nt * 32 + r;
-        btn_col[nt] = (TYPE == 2 && col < p.KN) ? p.btn[col] : 0;
-    }
-    float th_row[TM];
-#pragma unroll
-    for (int mt = 0; mt < TM; mt++) {
-        th_row[mt] = 0.f;
-        if (p.qy != nullptr) {
-            int n = (wave_m0 + mt * 32 + r) / (p.OH * p.OW);
-            n = n < p.N ? n : p.N - 1;  // rows past M are computed but not stored
-            th_row[mt] = p.out_ths[n];
-        }
-    }
 
     st.fetch(p, 0);
     st.stage(lds);
@@ -177,10 +165,10 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(4)
             i32x8 af[TM], bf[TN];
 #pragma unroll
             for (int mt = 0; mt < TM; mt++)
-                af[mt] = (APL == 2) ? expand_ternary<0>(a_w[w][0][mt], a_w[w][APL - 1][mt]) : expand_binary<0>(a_w[w][0][mt]);
+                af[mt] = (APL == 2) ? expand_ternary<0>(a_w[w][0][mt], a_w[w][APL - 1][mt], consts) : expand_binary<0>(a_w[w][0][mt], consts);
 #pragma unroll
             for (int nt = 0; nt < TN; nt++) {
-                bf[nt] = (BPL == 2) ? expand_ternary<1>(b_w[w][0][nt], b_w[w][BPL - 1][nt]) : expand_binary<1>(b_w[w][0][nt]);
+                bf[nt] = (BPL == 2) ? expand_ternary<1>(b_w[w][0][nt], b_w[w][BPL - 1][nt], consts) : expand_binary<1>(b_w[w][0][nt], consts);
                 if (TYPE == 2) b_nonzero[nt] += __builtin_popcount(b_w[w][BPL - 1][nt]);
             }
 #pragma unroll
@@ -195,6 +183,25 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(4)
     }
 
     // ---- epilogue: accumulator element 4*j + i of lane (kb, r) is C[8*j + 4*kb + i][r] -------
+    // btn of this lane's filters (BTN) and, for packed output, the threshold of row r of each 32-row
+    // tile; loaded here rather than before the loop because the registers they would hold through
+    // it push the 128x128 shape over its 128-register budget (requesting them early gained nothing)
+    int btn_col[TN];
+#pragma unroll
+    for (int nt = 0; nt < TN; nt++) {
+        const int col = wave_n0 + nt * 32 + r;
+        btn_col[nt] = (TYPE == 2 && col < p.KN) ? p.btn[col] : 0;
+    }
+    float th_row[TM];
+#pragma unroll
+    for (int mt = 0; mt < TM; mt++) {
+        th_row[mt] = 0.f;
+        if (p.qy != nullptr) {
+            int n = (wave_m0 + mt * 32 + r) / (p.OH * p.OW);
+            n = n < p.N ? n : p.N - 1;  // rows past M are computed but not stored
+            th_row[mt] = p.out_ths[n];
+        }
+    }
     const bool whole = wave_m0 + 32 * TM <= p.M && wave_n0 + 32 * TN <= p.KN;  // wave-uniform
     if (KS > 1) {
         // the KS waves hold partial sums of the same tile: exchange them through LDS; wave ks
