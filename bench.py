@@ -40,7 +40,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes moved by the ten conv launches of one headline step, from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE passes over `bench.py --profile` scaled by a 256 MiB copy
 # (profiles/quantize_conv_profile_sequence_traffic.txt).
-CONV_STEP_TRAFFIC_BYTES = 59132199
+CONV_STEP_TRAFFIC_BYTES = 59367722
 
 
 def valu_peak_tops(type):
@@ -54,10 +54,12 @@ def planning_peak_tops(type):
 
 
 def layer_bytes(N, layer, wbits=1):
-    """Algorithmic HBM bytes of one Conv2d call: X read, QW read, Y written."""
+    """Algorithmic HBM bytes of one Conv2d call: X read (only the pixels a 1x1 strided conv without
+    padding touches), QW read, Y written."""
     H, W, C, KN, KH, KW, p1, p2, s1, s2 = layer
     OH, OW = out_extent(H, p1, KH, s1), out_extent(W, p2, KW, s2)
-    return 4 * N * H * W * C + 8 * KN * KH * KW * ((C + 63) // 64) * wbits + 4 * N * OH * OW * KN
+    x_pixels = OH * OW if (KH, KW, p1, p2) == (1, 1, 0, 0) else H * W
+    return 4 * N * x_pixels * C + 8 * KN * KH * KW * ((C + 63) // 64) * wbits + 4 * N * OH * OW * KN
 
 
 def conv_kernel_bytes(N, layer, abits=1, wbits=1):
