@@ -56,7 +56,7 @@ hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream);
 // Matrix-core (FP4 MFMA) variant; shape picks the workgroup tile.  conv_mfma_exact() says whether K is
 // short enough for its fp32 accumulators to hold every partial sum exactly.
 bool conv_mfma_exact(const ConvArgs &args);
-int conv_mfma_shape(const ConvArgs &args);
+int conv_mfma_shape(int type, const ConvArgs &args);
 hipError_t launch_conv_mfma(int type, const ConvArgs &args, int shape, hipStream_t stream);
 hipError_t launch_conv_mfma_tnn(const ConvArgs &args, int shape, hipStream_t stream);
 hipError_t launch_conv_mfma_tbn(const ConvArgs &args, int shape, hipStream_t stream);

@@ -349,11 +349,14 @@ hipError_t launch_conv_mfma(int type, const ConvArgs &args, int shape, hipStream
 // N = 8 .. 256: the 128-row tiles win as soon as there is about one of them per CU (the 128x128 one
 // with short K they need about four per CU); below roughly 200 workgroups of 64x64 the launch is
 // latency-bound and the k-split 32x32 shape wins.
-int conv_mfma_shape(const ConvArgs &a)
+int conv_mfma_shape(int type, const ConvArgs &a)
 {
     auto tiles = [&](int bm, int bn) { return (long)((a.M + bm - 1) / bm) * ((a.KN + bn - 1) / bn); };
     const long enough = a.G >= 36 ? 300 : 1024;  // short K: the per-tile prologue and epilogue weigh more
     if (a.KN > 64 && a.G >= 18 && tiles(128, 128) >= enough) return 0;
+    // one tile of filters: 256 rows per workgroup halve the expansions per MFMA of the 128x64 shape (two-plane
+    // operands gain 20 %, BNN nothing)
+    if (a.KN <= 64 && type != 3 && tiles(256, 64) >= 1024) return 4;
     if (tiles(128, 64) >= enough) return 1;
     if (tiles(64, 64) >= 192 || a.qy != nullptr) return 2;  // the packed epilogue needs tiles 64 filters wide
     return 3;
@@ -363,13 +366,13 @@ hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream)
 {
     if (args.qy != nullptr) {  // packed output exists in the matrix-core kernel's 64-wide shapes only
         if (!conv_mfma_exact(args)) return hipErrorInvalidValue;
-        const int shape = (g_force_tm == 9 && g_force_ng >= 0 && g_force_ng <= 2) ? g_force_ng : conv_mfma_shape(args);
+        const int shape = (g_force_tm == 9 && g_force_ng >= 0 && g_force_ng != 3 && g_force_ng <= 4) ? g_force_ng : conv_mfma_shape(type, args);
         return launch_conv_mfma(type, args, shape, stream);
     }
-    if (g_force_tm == 9) return launch_conv_mfma(type, args, g_force_ng < 0 ? conv_mfma_shape(args) : g_force_ng, stream);
+    if (g_force_tm == 9) return launch_conv_mfma(type, args, g_force_ng < 0 ? conv_mfma_shape(type, args) : g_force_ng, stream);
     // default path: matrix cores; the popcount kernel takes over when K is too long for exact fp32
     // accumulation (and when a benchmark forces one of its tiles)
-    if (g_force_tm == 0 && conv_mfma_exact(args)) return launch_conv_mfma(type, args, conv_mfma_shape(args), stream);
+    if (g_force_tm == 0 && conv_mfma_exact(args)) return launch_conv_mfma(type, args, conv_mfma_shape(type, args), stream);
     switch (type) {
     case 0: return launch_type<0>(args, stream);
     case 1: return launch_type<1>(args, stream);

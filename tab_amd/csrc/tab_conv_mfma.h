@@ -368,7 +368,7 @@ hipError_t launch_mfma_shape(const ConvArgs &a, hipStream_t stream)
 }
 
 // shape: 0 = 128x128, 1 = 128x64, 2 = 64x64 (rows x filters per workgroup), 3 = 32x32 with the four
-// waves splitting every chunk of four words between them
+// waves splitting every chunk of four words between them, 4 = 256x64
 template <int TYPE>
 hipError_t launch_mfma_type(const ConvArgs &a, int shape, hipStream_t stream)
 {
@@ -376,6 +376,7 @@ hipError_t launch_mfma_type(const ConvArgs &a, int shape, hipStream_t stream)
     case 0: return launch_mfma_shape<TYPE, 2, 2, 2, 2>(a, stream);
     case 1: return launch_mfma_shape<TYPE, 4, 1, 1, 2>(a, stream);
     case 2: return launch_mfma_shape<TYPE, 2, 2, 1, 1, true>(a, stream);
+    case 4: return launch_mfma_shape<TYPE, 4, 1, 2, 2>(a, stream);
     case 3:
         if (a.PC % 8 == 0) return launch_mfma_tile<TYPE, 1, 1, 1, 1, 8, true, 4>(a, stream);
         if (a.PC % 4 == 0) return launch_mfma_tile<TYPE, 1, 1, 1, 1, 4, true, 4>(a, stream);
