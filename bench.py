@@ -167,8 +167,13 @@ def graph_time_ms(torch, fn, launches, replays=5):
     with torch.cuda.graph(graph):
         for _ in range(launches):
             fn()
-    graph.replay()
-    torch.cuda.synchronize()
+    # warm up for about 20 ms of replays: the first launches after an idle gap run at a lower clock
+    t0 = time.perf_counter()
+    while True:
+        graph.replay()
+        torch.cuda.synchronize()
+        if time.perf_counter() - t0 > 0.02:
+            break
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
     for _ in range(replays):

@@ -353,6 +353,16 @@ int conv_mfma_shape(int type, const ConvArgs &a)
 {
     auto tiles = [&](int bm, int bn) { return (long)((a.M + bm - 1) / bm) * ((a.KN + bn - 1) / bn); };
     const long enough = a.G >= 36 ? 300 : 1024;  // short K: the per-tile prologue and epilogue weigh more
+    // eight tiles per wave share each expanded operand between more MFMAs (the dearer operand gets the
+    // 4-tile side): +4-13 % for the types with a two-plane operand (nothing for BNN), but only when the
+    // launch is many rounds of these big tiles, or fits in one
+    if (a.G >= 36 && type != 3) {
+        const long big = tiles(256, 128);
+        if (big >= 2560 || (big >= 300 && big <= 512)) {
+            if (type == 1 && a.KN >= 256) return 6;
+            if (type != 1 && a.KN >= 128) return 5;
+        }
+    }
     if (a.KN > 64 && a.G >= 18 && tiles(128, 128) >= enough) return 0;
     // one tile of filters: 256 rows per workgroup halve the expansions per MFMA of the 128x64 shape (two-plane
     // operands gain 20 %, BNN nothing)
@@ -366,7 +376,7 @@ hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream)
 {
     if (args.qy != nullptr) {  // packed output exists in the matrix-core kernel's 64-wide shapes only
         if (!conv_mfma_exact(args)) return hipErrorInvalidValue;
-        const int shape = (g_force_tm == 9 && g_force_ng >= 0 && g_force_ng != 3 && g_force_ng <= 4) ? g_force_ng : conv_mfma_shape(type, args);
+        const int shape = (g_force_tm == 9 && g_force_ng >= 0 && g_force_ng != 3 && g_force_ng <= 6) ? g_force_ng : conv_mfma_shape(type, args);
         return launch_conv_mfma(type, args, shape, stream);
     }
     if (g_force_tm == 9) return launch_conv_mfma(type, args, g_force_ng < 0 ? conv_mfma_shape(type, args) : g_force_ng, stream);

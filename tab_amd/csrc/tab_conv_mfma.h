@@ -81,10 +81,12 @@ __device__ __forceinline__ i32x8 expand_ternary(uint32_t s, uint32_t z, const Ex
     return r;
 }
 
-// waves_per_eu(4): at most 128 registers, i.e. four workgroups per CU; the 128x128 shape otherwise takes
-// 136-152 (64 of them accumulators) and runs three, measured 3-7 % slower.
+// waves_per_eu: the shapes with four MFMA tiles per wave are capped at 128 registers, i.e. four
+// workgroups per CU (the 128x128 shape otherwise takes 136-152, 64 of them accumulators, and runs
+// three, measured 3-7 % slower); 256-row tiles need the state of more staged rows and get 168
+// (three workgroups), eight tiles per wave 256 (two).
 template <int TYPE, int WM, int WN, int TM, int TN, int KCH, bool INTAP, int KS = 1>
-__global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(4))) void conv_mfma(const ConvArgs p)
+__global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM * TN > 4 ? 2 : (WM * TM > 4 ? 3 : 4)))) void conv_mfma(const ConvArgs p)
 {
     static_assert(WM * WN * KS * 64 == kConvThreads, "four waves");
     static_assert(KCH % KS == 0 && (KS == 1 || (TM == 1 && TN == 1)), "k-split waves share one 32x32 tile");
@@ -368,7 +370,8 @@ hipError_t launch_mfma_shape(const ConvArgs &a, hipStream_t stream)
 }
 
 // shape: 0 = 128x128, 1 = 128x64, 2 = 64x64 (rows x filters per workgroup), 3 = 32x32 with the four
-// waves splitting every chunk of four words between them, 4 = 256x64
+// waves splitting every chunk of four words between them, 4 = 256x64, 5 = 256x128 and 6 = 128x256
+// (eight MFMA tiles per wave: fewer operand expansions per MFMA, half the occupancy)
 template <int TYPE>
 hipError_t launch_mfma_type(const ConvArgs &a, int shape, hipStream_t stream)
 {
@@ -377,6 +380,8 @@ hipError_t launch_mfma_type(const ConvArgs &a, int shape, hipStream_t stream)
     case 1: return launch_mfma_shape<TYPE, 4, 1, 1, 2>(a, stream);
     case 2: return launch_mfma_shape<TYPE, 2, 2, 1, 1, true>(a, stream);
     case 4: return launch_mfma_shape<TYPE, 4, 1, 2, 2>(a, stream);
+    case 5: return launch_mfma_shape<TYPE, 2, 2, 4, 2>(a, stream);
+    case 6: return launch_mfma_shape<TYPE, 2, 2, 2, 4>(a, stream);
     case 3:
         if (a.PC % 8 == 0) return launch_mfma_tile<TYPE, 1, 1, 1, 1, 8, true, 4>(a, stream);
         if (a.PC % 4 == 0) return launch_mfma_tile<TYPE, 1, 1, 1, 1, 4, true, 4>(a, stream);

@@ -65,7 +65,7 @@ def test_packed_out(type, case, out_bits):
         _packed_out_case(type, *case, out_bits, kind, seed=type + out_bits)
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 4])
+@pytest.mark.parametrize("tile", [0, 1, 2, 4, 5, 6])
 @pytest.mark.parametrize("type", [0, 3])
 def test_packed_out_every_tile(type, tile, restore_kernel_choice):
     tab_amd.set_conv_kernel(tab_amd.CONV_MATRIX, tile)
