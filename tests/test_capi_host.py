@@ -66,6 +66,30 @@ def test_c_abi_rejects_bad_arguments_without_launching():
     assert lib.tab_conv2d_packed(p, p, None, 2, 1, 1, 1, 1, 1, 8, 8, 64, 4, 3, 3, p, None) == -1
     with pytest.raises(_capi.TabError, match="TAB_ERR_BAD_ARGUMENT"):
         _capi.check(lib, lib.tab_quantize(p, p, 0, 1, 1, 1, 64, p, p, None))
+    # packed output: bit width, thresholds, output pointer, alignment of a 2-bit element
+    out = lambda **kw: lib.tab_conv2d_packed_out(  # noqa: E731
+        p, p, p, 3, 1, 1, 1, 1, 1, 8, 8, 64, 4, 3, 3, kw.get("ths", p), kw.get("bits", 1), kw.get("qy", p), None)
+    assert out(bits=3) == -1 and b"out_bitwidth" in lib.tab_last_error()
+    assert out(ths=None) == -1
+    assert out(qy=None) == -1
+    assert out(qy=p + 8, bits=2) == -1 and b"aligned" in lib.tab_last_error()
+    # threshold: workspace
+    assert lib.tab_threshold_workspace_bytes(0, 10) == 0
+    assert lib.tab_threshold(p, 4, 100, ctypes.c_float(0.7), p, None, 0, None) == -3
+    # a packed image too large for 32-bit offsets inside one workgroup
+    assert lib.tab_conv2d_packed(p, p, p, 3, 0, 0, 1, 1, 1, 30000, 30000, 64, 4, 1, 1, p, None) == -2
+    assert b"32-bit" in lib.tab_last_error()
+
+
+def test_set_conv_kernel_validates_without_a_gpu():
+    lib = _capi.load()
+    try:
+        for kernel, tile, ok in [(0, -1, True), (1, -1, True), (1, 6, True), (1, 7, False), (2, 2, True), (2, 3, False),
+                                 (0, 0, False), (3, -1, False)]:
+            assert (lib.tab_set_conv_kernel(kernel, tile) == 0) == ok, (kernel, tile)
+        assert b"no conv kernel" in lib.tab_last_error()
+    finally:
+        assert lib.tab_set_conv_kernel(0, -1) == 0
 
 
 def test_python_mirror_names_and_input_checks():

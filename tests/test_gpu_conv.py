@@ -166,11 +166,11 @@ def test_full_size_sweep_point_properties():
     must equal the same images inside the full batch; the first and the last image are compared
     with the oracle; and every output obeys |y| <= KH*KW*C and, for BNN, y = NUM (mod 2)."""
     N, H, W, C, KN = 256, 28, 28, 512, 512
-    print("[case] full-size sweep point N=256 28x28x512->512 3x3 BNN/TNN", flush=True)
+    print("[case] full-size sweep point N=256 28x28x512->512 3x3, four types", flush=True)
     g = torch.Generator("cuda").manual_seed(0)
     x = torch.randn((N, H, W, C), generator=g, device="cuda")
     w = torch.randn((KN, 3, 3, C), generator=g, device="cuda")
-    for type in (3, 0):
+    for type in (3, 0, 1, 2):  # every type takes its own tile shape at this size
         ab, wb = act_bits(type), weight_bits(type)
         x_ths = (0.7 * x.abs().reshape(N, -1).mean(dim=1)).contiguous() if ab == 2 else torch.zeros(N, device="cuda")
         w_ths = (0.7 * w.abs().reshape(KN, -1).mean(dim=1)).contiguous() if wb == 2 else torch.zeros(KN, device="cuda")
