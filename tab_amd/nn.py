@@ -8,7 +8,7 @@ Inference only (the operators have no backward).
 import torch
 from torch import nn
 
-from . import BNN, BTN, TBN, TNN, Conv2d, Quantize, Threshold, out_shape
+from . import BNN, BTN, TBN, TNN, Conv2d, Conv2dPacked, Conv2dPackedOut, Quantize, Threshold, out_shape
 
 _ACT_BITS = {TNN: 2, TBN: 2, BTN: 1, BNN: 1}
 _WEIGHT_BITS = {TNN: 2, TBN: 1, BTN: 2, BNN: 1}
@@ -95,3 +95,57 @@ class TABLinear(nn.Module):
     def forward(self, x):
         N, F = x.shape
         return self.conv(x.reshape(N, 1, 1, F)).reshape(N, self.conv.out_channels)
+
+
+class TABPackedChain(nn.Module):
+    """A stack of TABConv2d layers run packed-in / packed-out: the input is quantized once, every
+    layer but the last writes its output already thresholded and packed for the next layer (no fp32
+    activation between layers), the last one returns fp32.  A layer's output channels must be the
+    next layer's input channels.
+
+    The threshold applied to a layer's output is the next layer's activation threshold: 0 when the
+    next layer takes binary activations (types BTN, BNN) - then the chain returns exactly what
+    calling the layers one after the other returns - and, when it takes ternary activations, the
+    calibrated constant given in `ternary_thresholds[i]` for layer i+1 (the per-image
+    `act_scale * mean|y|` of an unchained TABConv2d needs the fp32 tensor this class avoids)."""
+
+    def __init__(self, layers, ternary_thresholds=None, data_format="NCHW"):
+        super().__init__()
+        self.layers = nn.ModuleList(layers)
+        if not self.layers:
+            raise ValueError("at least one layer")
+        for a, b in zip(self.layers[:-1], self.layers[1:]):
+            if a.out_channels != b.in_channels:
+                raise ValueError(f"{a.out_channels} output channels feed a layer with {b.in_channels} input channels")
+        self.ternary_thresholds = dict(ternary_thresholds or {})
+        for i, layer in enumerate(self.layers[1:], start=1):
+            if _ACT_BITS[layer.conv_type] == 2 and i not in self.ternary_thresholds:
+                raise ValueError(f"layer {i} takes ternary activations: give ternary_thresholds[{i}]")
+        if data_format not in ("NCHW", "NHWC"):
+            raise ValueError("data_format must be 'NCHW' or 'NHWC'")
+        self.data_format = data_format
+
+    def forward(self, x):
+        if self.data_format == "NCHW":
+            N, C, H, W = x.shape
+            x = x.permute(0, 2, 3, 1)
+        else:
+            N, H, W, C = x.shape
+        first = self.layers[0]
+        if C != first.in_channels:
+            raise RuntimeError(f"expected {first.in_channels} input channels, got {C}")
+        x = x.to(torch.float32).contiguous()
+        bits = _ACT_BITS[first.conv_type]
+        ths = Threshold(x, N, first.act_scale) if bits == 2 else torch.zeros(N, dtype=torch.float32, device=x.device)
+        q, _ = Quantize(x, ths, bits, N, H, W, C)
+        for i, layer in enumerate(self.layers):
+            (KH, KW), (s1, s2), (p1, p2) = layer.kernel_size, layer.stride, layer.padding
+            args = (layer.conv_type, p1, p2, s1, s2, N, H, W, layer.in_channels, layer.out_channels, KH, KW)
+            OH, OW = out_shape(H, W, KH, KW, p1, p2, s1, s2)
+            if i + 1 == len(self.layers):
+                y = Conv2dPacked(q, layer.QW, layer.BTN_W, *args).view(N, OH, OW, layer.out_channels)
+                return y.permute(0, 3, 1, 2) if self.data_format == "NCHW" else y
+            next_bits = _ACT_BITS[self.layers[i + 1].conv_type]
+            out_ths = torch.full((N,), float(self.ternary_thresholds.get(i + 1, 0.0)), dtype=torch.float32, device=x.device)
+            q = Conv2dPackedOut(q, layer.QW, layer.BTN_W, *args, out_ths, next_bits)
+            H, W = OH, OW

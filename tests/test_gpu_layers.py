@@ -78,3 +78,42 @@ def test_linear_module_is_integer_dot_product():
     sx = torch.where(x < 0, -1.0, 1.0)
     sw = torch.where(w < 0, -1.0, 1.0)
     assert torch.equal(y.cpu(), sx @ sw.t())
+
+
+def test_packed_chain_equals_layer_by_layer():
+    """Three binary-activation layers (BNN, BTN, BNN) chained packed-to-packed return exactly what
+    the same modules return one after the other (threshold 0 on both paths), and a ternary layer in
+    the middle with a calibrated threshold matches the oracle's conv -> quantize -> conv."""
+    from tab_amd.nn import TABPackedChain
+
+    g = torch.Generator("cpu").manual_seed(3)
+    x = torch.randn((3, 64, 12, 12), generator=g)
+    w1 = torch.randn((128, 64, 3, 3), generator=g)
+    w2 = torch.randn((96, 128, 3, 3), generator=g)
+    w3 = torch.randn((40, 96, 1, 1), generator=g)
+    l1 = TABConv2d.from_float(w1, tab_amd.BNN, stride=1, padding=1)
+    l2 = TABConv2d.from_float(w2, tab_amd.BTN, stride=2, padding=1)
+    l3 = TABConv2d.from_float(w3, tab_amd.BNN)
+    print("[case] TABPackedChain BNN -> BTN -> BNN", flush=True)
+    chain = TABPackedChain([l1, l2, l3])
+    got = chain(x.cuda())
+    want = l3(l2(l1(x.cuda())))
+    torch.cuda.synchronize()
+    assert got.shape == want.shape and torch.equal(got, want)
+
+    # a ternary-activation layer second: its input threshold is the constant given to the chain
+    print("[case] TABPackedChain BNN -> TNN with a calibrated threshold", flush=True)
+    t2 = TABConv2d.from_float(w2, tab_amd.TNN, stride=1, padding=1)
+    chain = TABPackedChain([l1, t2], ternary_thresholds={1: 24.0}, data_format="NHWC")
+    xh = x.permute(0, 2, 3, 1).contiguous()
+    got = chain(xh.cuda()).cpu().numpy()
+    N, H, W = 3, 12, 12
+    zeros = np.zeros(N, dtype=np.float32)
+    y1 = oracle.conv2d(xh.numpy(), l1.QW.cpu().numpy(), zeros, l1.BTN_W.cpu().numpy(), 3, 1, 1, 1, 1, N, H, W, 64, 128, 3, 3)
+    y2 = oracle.conv2d(np.ascontiguousarray(y1).reshape(N, H, W, 128), t2.QW.cpu().numpy(), np.full(N, 24.0, np.float32),
+                       t2.BTN_W.cpu().numpy(), 0, 1, 1, 1, 1, N, H, W, 128, 96, 3, 3)
+    assert np.array_equal(got.reshape(-1), np.ascontiguousarray(y2).reshape(-1))
+    with pytest.raises(ValueError, match="ternary_thresholds"):
+        TABPackedChain([l1, t2])
+    with pytest.raises(ValueError, match="input channels"):
+        TABPackedChain([l1, l3])
