@@ -48,7 +48,7 @@ def lib():
         L.oracle_num_threads.restype = _int
         L.oracle_out_extent.restype = _int
         L.oracle_out_extent.argtypes = [_int] * 4
-        for name in ("oracle_quantize_ternary", "oracle_quantize_binary"):
+        for name in ("oracle_quantize_ternary", "oracle_quantize_binary", "oracle_quantize_drf", "oracle_quantize_rtn"):
             getattr(L, name).argtypes = [_c_f32, _c_f32, _int, _int, _int, _int, _c_i64]
             getattr(L, name).restype = None
         L.oracle_btn_weight.argtypes = [_c_i64, _int, _long, _c_i32]
@@ -61,8 +61,12 @@ def lib():
         L.oracle_gemm_tbn.argtypes = [_c_i64, _c_i64, _long, _int, _int, _c_i32]
         L.oracle_gemm_btn.argtypes = [_c_i64, _c_i64, _c_i32, _long, _int, _int, _c_i32]
         L.oracle_gemm_bnn.argtypes = [_c_i64, _c_i64, _long, _int, _int, _int, _c_i32]
+        L.oracle_gemm_drf.argtypes = [_c_i64, _c_i64, _long, _int, _int, _c_i32]
+        L.oracle_gemm_rtn.argtypes = [_c_i64, _c_i64, _long, _int, _int, _c_i32]
         L.oracle_conv2d.argtypes = [_c_f32, _c_i64, _c_f32, _c_i32] + [_int] * 12 + [_c_f32]
         L.oracle_conv2d.restype = _int
+        L.oracle_conv2d_packed.argtypes = [_c_i64, _c_i64, _c_i32] + [_int] * 12 + [_c_f32]
+        L.oracle_conv2d_packed.restype = _int
         _lib = L
     return _lib
 
@@ -107,6 +111,36 @@ def quantize(x, ths, bitwidth, N, H, W, C):
     return qx, btn
 
 
+TYPE_DRF, TYPE_RTN = 4, 5  # the CPU-only types of TAB_Conv (TAB_CPU.cpp:332-383)
+
+
+def words_per_pixel(type, C, operand):
+    """int64 words per pixel of operand 'a' (activation) or 'w' (weight) for conv type 0..5."""
+    if type == TYPE_RTN:
+        return (C + 31) // 32
+    if type == TYPE_DRF:
+        return 2 * packed_channels(C)
+    two_planes = type < 2 if operand == "a" else type in (0, 2)
+    return packed_channels(C) * (2 if two_planes else 1)
+
+
+def quantize_format(x, ths, type, N, H, W, C):
+    """Packers of the two CPU-only types: 4 -> DoReFa levels (N,H,W,PC,2), 5 -> RTN fields
+    (N,H,W,ceil(C/32)).  The reference defines the layouts (through its GEMMs) but no
+    quantizer; the value rules are documented in tab_oracle.c."""
+    x, ths = _f32(x), _f32(ths)
+    assert x.size == N * H * W * C and ths.size >= N
+    if type == TYPE_DRF:
+        qx = np.empty((N, H, W, packed_channels(C), 2), dtype=np.int64)
+        lib().oracle_quantize_drf(_ptr(x, _c_f32), _ptr(ths, _c_f32), N, H, W, C, _ptr(qx, _c_i64))
+    elif type == TYPE_RTN:
+        qx = np.empty((N, H, W, (C + 31) // 32), dtype=np.int64)
+        lib().oracle_quantize_rtn(_ptr(x, _c_f32), _ptr(ths, _c_f32), N, H, W, C, _ptr(qx, _c_i64))
+    else:
+        raise ValueError("type must be 4 or 5")
+    return qx
+
+
 def pad(a, N, H, W, D, p1, p2):
     a = _i64(a)
     y = np.empty((N, H + 2 * p1, W + 2 * p2, D), dtype=np.int64)
@@ -123,7 +157,7 @@ def img2row(a, N, PH, PW, D, KH, KW, s1, s2):
 
 
 def gemm(type, a, b, M, N, K, btn=None, NUM=0):
-    """One of the four popcount GEMMs (TAB_CPU.cpp:242-328); returns int32 [M,N]."""
+    """One of the six popcount GEMMs (TAB_CPU.cpp:242-383); returns int32 [M,N]."""
     a, b = _i64(a), _i64(b)
     y = np.empty((M, N), dtype=np.int32)
     L = lib()
@@ -136,8 +170,12 @@ def gemm(type, a, b, M, N, K, btn=None, NUM=0):
         L.oracle_gemm_btn(_ptr(a, _c_i64), _ptr(b, _c_i64), _ptr(btn, _c_i32), M, N, K, _ptr(y, _c_i32))
     elif type == 3:
         L.oracle_gemm_bnn(_ptr(a, _c_i64), _ptr(b, _c_i64), M, N, K, NUM, _ptr(y, _c_i32))
+    elif type == TYPE_DRF:
+        L.oracle_gemm_drf(_ptr(a, _c_i64), _ptr(b, _c_i64), M, N, K, _ptr(y, _c_i32))
+    elif type == TYPE_RTN:
+        L.oracle_gemm_rtn(_ptr(a, _c_i64), _ptr(b, _c_i64), M, N, K, _ptr(y, _c_i32))
     else:
-        raise ValueError("type must be 0..3")
+        raise ValueError("type must be 0..5")
     return y
 
 
@@ -150,6 +188,21 @@ def conv2d(x, qw, ths, btn, type, p1, p2, s1, s2, N, H, W, C, KN, KH, KW):
                              type, p1, p2, s1, s2, N, H, W, C, KN, KH, KW, _ptr(y, _c_f32))
     if rc != 0:
         raise ValueError("oracle_conv2d rejected the arguments")
+    return y
+
+
+def conv2d_packed(qx, qw, btn, type, p1, p2, s1, s2, N, H, W, C, KN, KH, KW):
+    """Conv2d on a packed activation (pad, im2row, GEMM), types 0..5; fp32 (N,KN,OH,OW)."""
+    qx, qw = _i64(qx), _i64(qw)
+    btn = _i32(btn if btn is not None else np.zeros(KN))
+    assert qx.size == N * H * W * words_per_pixel(type, C, "a")
+    assert qw.size == KN * KH * KW * words_per_pixel(type, C, "w")
+    OH, OW = out_extent(H, p1, KH, s1), out_extent(W, p2, KW, s2)
+    y = np.empty((N, KN, OH, OW), dtype=np.float32)
+    rc = lib().oracle_conv2d_packed(_ptr(qx, _c_i64), _ptr(qw, _c_i64), _ptr(btn, _c_i32), type, p1, p2, s1, s2,
+                                    N, H, W, C, KN, KH, KW, _ptr(y, _c_f32))
+    if rc != 0:
+        raise ValueError("oracle_conv2d_packed rejected the arguments")
     return y
 
 
@@ -170,6 +223,9 @@ def ref():
         R.ref_gemm_tbn.argtypes = [_c_i64, _c_i64, _int, _int, _int, _c_i32]
         R.ref_gemm_btn.argtypes = [_c_i64, _c_i64, _c_i32, _int, _int, _int, _c_i32]
         R.ref_gemm_bnn.argtypes = [_c_i64, _c_i64, _int, _int, _int, _int, _c_i32]
+        if hasattr(R, "ref_gemm_drf"):
+            R.ref_gemm_drf.argtypes = [_c_i64, _c_i64, _int, _int, _int, _c_i32]
+            R.ref_gemm_rtn.argtypes = [_c_i64, _c_i64, _int, _int, _int, _c_i32]
         R.ref_img2row_3x3.argtypes = [_c_i64] + [_int] * 8 + [_c_i64]
         R.ref_ternarize_nchw.argtypes = [_c_f32, _int, _int, _c_f32] + [_int] * 4 + [_c_i64]
         R.ref_binarize_nchw.argtypes = [_c_f32, _int, _int] + [_int] * 4 + [_c_i64]
@@ -188,8 +244,12 @@ def ref_gemm(type, a, b, M, N, K, btn=None, NUM=0):
     elif type == 2:
         btn = _i32(btn).copy()
         R.ref_gemm_btn(_ptr(a, _c_i64), _ptr(b, _c_i64), _ptr(btn, _c_i32), M, N, K, _ptr(y, _c_i32))
-    else:
+    elif type == 3:
         R.ref_gemm_bnn(_ptr(a, _c_i64), _ptr(b, _c_i64), M, N, K, NUM, _ptr(y, _c_i32))
+    elif type == TYPE_DRF:
+        R.ref_gemm_drf(_ptr(a, _c_i64), _ptr(b, _c_i64), M, N, K, _ptr(y, _c_i32))
+    else:
+        R.ref_gemm_rtn(_ptr(a, _c_i64), _ptr(b, _c_i64), M, N, K, _ptr(y, _c_i32))
     return y
 
 

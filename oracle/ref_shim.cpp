@@ -40,6 +40,18 @@ void ref_gemm_bnn(int64_t *a, int64_t *b, int M, int N, int K, int NUM, int32_t 
     std::memcpy(y, r.data(), sizeof(int) * r.size());
 }
 
+// TAB_CPU.cpp:332-383, the CPU-only types 4 (DoReFa 2-bit) and 5 (RTN).
+void ref_gemm_drf(int64_t *a, int64_t *b, int M, int N, int K, int32_t *y)
+{
+    std::vector<int> r = DRFGEMM_baseline(a, b, M, N, K);
+    std::memcpy(y, r.data(), sizeof(int) * r.size());
+}
+void ref_gemm_rtn(int64_t *a, int64_t *b, int M, int N, int K, int32_t *y)
+{
+    std::vector<int> r = RTNGEMM_baseline(a, b, M, N, K);
+    std::memcpy(y, r.data(), sizeof(int) * r.size());
+}
+
 // TAB_CPU.h:27-63.  x is [N][H][W][D] packed words (already padded); rows is
 // [N*OH*OW][KH*KW*D].  The routine copies exactly three kernel rows, so KH must be 3.
 void ref_img2row_3x3(int64_t *x, int N, int D, int H, int W, int KH, int KW, int s1, int s2,

@@ -12,6 +12,7 @@
  *   - zero padding of packed words   TAB_GEMM.cuh:73-89, TAB_CPU.cpp:39,155
  *   - im2row, K order (kh,kw,c)  TAB_GEMM.cuh:92-115, TAB_CPU.h:27-63
  *   - the four popcount GEMMs    TAB_CPU.cpp:242-328 (== TAB_GEMM.cu:25-147)
+ *   - the two CPU-only GEMMs     TAB_CPU.cpp:332-383 (type 4 DoReFa 2-bit, type 5 RTN)
  *   - the conv pipeline          TAB_GEMM.cu:325-527, TAB_CPU.cpp:507-614
  *
  * Pinning (what checks each function independently of this file's own formulas):
@@ -24,7 +25,15 @@
  *                   ternarizer compiled from /root/reference on single-image inputs;
  *   btn           : equals the number of nonzero ternary weights per filter;
  *   conv2d        : torch.nn.functional.conv2d on the dequantised {-1,0,+1} tensors
- *                   (padding value 0 for ternary, +1 for binary activations).
+ *                   (padding value 0 for ternary, +1 for binary activations);
+ *   gemm_drf/rtn  : bit-exact against DRFGEMM_baseline / RTNGEMM_baseline compiled from
+ *                   /root/reference (oracle/_ref, golden fixtures), and against integer dot
+ *                   products of the decoded values (levels 0..3; ternary fields);
+ *   quantize_drf, quantize_rtn : PARITY UNPINNED.  The reference has no quantizer for these
+ *                   two types (TAB_Conv names Parallel_Binarize_NCHW and
+ *                   Parallel_Ternarize_RTN, TAB_CPU.cpp:522,527, which no file defines); the
+ *                   word layouts follow from the GEMMs, the value rules are this build's
+ *                   own and are only checked against brute-force closed forms.
  */
 #include <stdint.h>
 #include <stdlib.h>
@@ -137,6 +146,70 @@ void oracle_quantize_binary(const float *x, const float *ths, int N, int H, int 
             for (int c = w * WORD_BITS; c < c_hi; c++)
                 if (src[c] < t) neg |= (uint64_t)1 << (c - w * WORD_BITS);
             dst[w] = neg;
+        }
+    }
+}
+
+/*
+ * DoReFa 2-bit levels (type 4).  Word layout from DRFGEMM_baseline (TAB_CPU.cpp:345-354):
+ * [pixel][PC][2] with plane 0 the weight-2 bit and plane 1 the weight-1 bit of a level 0..3.
+ * Value rule (this build's own, the reference defines none): a uniform quantizer with step
+ * t = ths[n], level = (v >= 0.5t) + (v >= 1.5t) + (v >= 2.5t), each bound rounded to fp32;
+ * NaN gives level 0.
+ */
+void oracle_quantize_drf(const float *x, const float *ths, int N, int H, int W, int C,
+                         int64_t *qx)
+{
+    const int PC = packed_channels(C);
+    const long pix_per_img = (long)H * W;
+#pragma omp parallel for schedule(static)
+    for (long p = 0; p < (long)N * pix_per_img; p++) {
+        const float t = ths[p / pix_per_img];
+        const float b1 = 0.5f * t, b2 = 1.5f * t, b3 = 2.5f * t;
+        const float *src = x + p * C;
+        uint64_t *dst = (uint64_t *)qx + p * PC * 2;
+        for (int w = 0; w < PC; w++) {
+            uint64_t hi = 0, lo = 0;
+            const int c_hi = (w + 1) * WORD_BITS < C ? (w + 1) * WORD_BITS : C;
+            for (int c = w * WORD_BITS; c < c_hi; c++) {
+                const float v = src[c];
+                const int level = (v >= b1) + (v >= b2) + (v >= b3);
+                hi |= (uint64_t)(level >> 1) << (c - w * WORD_BITS);
+                lo |= (uint64_t)(level & 1) << (c - w * WORD_BITS);
+            }
+            dst[2 * w + 0] = hi;
+            dst[2 * w + 1] = lo;
+        }
+    }
+}
+
+/*
+ * RTN ternary fields (type 5).  Word layout from RTNGEMM_baseline (TAB_CPU.cpp:364-379, mask
+ * 0x5555...) and TAB_CPU.cpp:520-521 (32 channels per word): channel c sits in word c/32 as a
+ * 2-bit field, bit 2*(c%32) = nonzero marker, bit 2*(c%32)+1 = sign marker.  Value rule: the
+ * ternarizer's (v > t -> +1, else v < -t -> -1, TAB_GEMM.cu:184-192), this build's choice.
+ */
+void oracle_quantize_rtn(const float *x, const float *ths, int N, int H, int W, int C,
+                         int64_t *qx)
+{
+    const int PC = (C + 31) / 32;
+    const long pix_per_img = (long)H * W;
+#pragma omp parallel for schedule(static)
+    for (long p = 0; p < (long)N * pix_per_img; p++) {
+        const float t = ths[p / pix_per_img];
+        const float *src = x + p * C;
+        uint64_t *dst = (uint64_t *)qx + p * PC;
+        for (int w = 0; w < PC; w++) {
+            uint64_t word = 0;
+            const int c_hi = (w + 1) * 32 < C ? (w + 1) * 32 : C;
+            for (int c = w * 32; c < c_hi; c++) {
+                const float v = src[c];
+                uint64_t field = 0;
+                if (v > t) field = 1;
+                else if (v < -t) field = 3;
+                word |= field << (2 * (c - w * 32));
+            }
+            dst[w] = word;
         }
     }
 }
@@ -259,6 +332,46 @@ ALWAYS_INLINE void body_bnn(const uint64_t *a, const uint64_t *b, long m0, long 
         }
 }
 
+/* DoReFa 2-bit (TAB_CPU.cpp:332-358): y = sum over k of (2*a0 + a1) * (2*b0 + b1) per bit */
+ALWAYS_INLINE void body_drf(const uint64_t *a, const uint64_t *b, long m0, long m1, int N,
+                            int K, int32_t *y)
+{
+    for (long m = m0; m < m1; m++)
+        for (int n = 0; n < N; n++) {
+            const uint64_t *ra = a + m * K * 2, *rb = b + (long)n * K * 2;
+            int32_t hh = 0, cross = 0, ll = 0;
+            for (int k = 0; k < K; k++) {
+                hh += __builtin_popcountll(ra[2 * k] & rb[2 * k]);
+                cross += __builtin_popcountll(ra[2 * k + 1] & rb[2 * k]);
+                cross += __builtin_popcountll(ra[2 * k] & rb[2 * k + 1]);
+                ll += __builtin_popcountll(ra[2 * k + 1] & rb[2 * k + 1]);
+            }
+            y[m * N + n] = 4 * hh + 2 * cross + ll;
+        }
+}
+
+/*
+ * RTN (TAB_CPU.cpp:362-383): 2-bit fields, even bit = nonzero, odd bit = sign;
+ * y = popcount(both nonzero) - 2 * popcount(both nonzero and signs differ).
+ */
+ALWAYS_INLINE void body_rtn(const uint64_t *a, const uint64_t *b, long m0, long m1, int N,
+                            int K, int32_t *y)
+{
+    const uint64_t even = 0x5555555555555555ull;
+    for (long m = m0; m < m1; m++)
+        for (int n = 0; n < N; n++) {
+            const uint64_t *ra = a + m * K, *rb = b + (long)n * K;
+            int32_t nonzero = 0, negative = 0;
+            for (int k = 0; k < K; k++) {
+                const uint64_t both = ra[k] & rb[k] & even;
+                const uint64_t differ = (ra[k] ^ rb[k]) >> 1;
+                nonzero += __builtin_popcountll(both);
+                negative += __builtin_popcountll(differ & both);
+            }
+            y[m * N + n] = nonzero - 2 * negative;
+        }
+}
+
 /*
  * One exported entry per type.  VARIANTS expands the row-range body once per ISA level;
  * the exported function splits the M rows into contiguous blocks, one per OpenMP thread
@@ -300,6 +413,11 @@ VARIANTS(btn, (const uint64_t *a, const uint64_t *b, const int32_t *btn, long m0
 VARIANTS(bnn, (const uint64_t *a, const uint64_t *b, long m0, long m1, int N, int K, int NUM, int32_t *y),
          (a, b, m0, m1, N, K, NUM, y))
 
+VARIANTS(drf, (const uint64_t *a, const uint64_t *b, long m0, long m1, int N, int K, int32_t *y),
+         (a, b, m0, m1, N, K, y))
+VARIANTS(rtn, (const uint64_t *a, const uint64_t *b, long m0, long m1, int N, int K, int32_t *y),
+         (a, b, m0, m1, N, K, y))
+
 void oracle_gemm_tnn(const int64_t *a, const int64_t *b, long M, int N, int K, int32_t *y)
 {
 #pragma omp parallel
@@ -339,48 +457,90 @@ void oracle_gemm_bnn(const int64_t *a, const int64_t *b, long M, int N, int K, i
     }
 }
 
-/*
- * Whole Conv2d call (TAB_GEMM.cu:325-527): quantize the activation by type
- * (ternary for 0/1, binary for 2/3; 419-426), zero-pad, im2row, GEMM with
- * M=N*OH*OW, K=KH*KW*PC, NUM=KH*KW*C (509).  y holds the int result converted to
- * fp32 at y[m*KN + kn], i.e. (n,oh,ow,kn) memory order (TAB_GEMM.cu:53,526).
- * Returns 0, or -1 on a bad type / empty output / allocation failure.
- */
-int oracle_conv2d(const float *x, const int64_t *qw, const float *ths, const int32_t *btn,
-                  int type, int p1, int p2, int s1, int s2, int N, int H, int W, int C, int KN,
-                  int KH, int KW, float *y)
+void oracle_gemm_drf(const int64_t *a, const int64_t *b, long M, int N, int K, int32_t *y)
 {
-    if (type < 0 || type > 3 || s1 < 1 || s2 < 1) return -1;
-    const int PC = packed_channels(C);
-    const int D = (type < 2) ? PC * 2 : PC; /* activation words per pixel */
+#pragma omp parallel
+    {
+        long m0, m1;
+        row_block(M, &m0, &m1);
+        run_drf((const uint64_t *)a, (const uint64_t *)b, m0, m1, N, K, y);
+    }
+}
+void oracle_gemm_rtn(const int64_t *a, const int64_t *b, long M, int N, int K, int32_t *y)
+{
+#pragma omp parallel
+    {
+        long m0, m1;
+        row_block(M, &m0, &m1);
+        run_rtn((const uint64_t *)a, (const uint64_t *)b, m0, m1, N, K, y);
+    }
+}
+
+/*
+ * Conv2d on an activation that is already packed, all six types of the CPU path
+ * (TAB_CPU.cpp:507-614): zero-pad, im2row, GEMM.  Words per pixel D: 2*PC for types 0, 1, 4
+ * (two planes), PC for 2, 3 (PC = ceil(C/64)), ceil(C/32) for type 5 (TAB_CPU.cpp:520-521).
+ * Padded taps are zero words: value 0 for types 0, 1, 4, 5 and +1 for binary activations.
+ */
+int oracle_conv2d_packed(const int64_t *qx, const int64_t *qw, const int32_t *btn, int type,
+                         int p1, int p2, int s1, int s2, int N, int H, int W, int C, int KN,
+                         int KH, int KW, float *y)
+{
+    if (type < 0 || type > 5 || s1 < 1 || s2 < 1) return -1;
+    const int PC = type == 5 ? (C + 31) / 32 : packed_channels(C);
+    const int D = (type < 2 || type == 4) ? PC * 2 : PC;
     const int PH = H + 2 * p1, PW = W + 2 * p2;
     const int OH = oracle_out_extent(H, p1, KH, s1), OW = oracle_out_extent(W, p2, KW, s2);
     if (OH < 1 || OW < 1) return -1;
     const long M = (long)N * OH * OW;
     const int K = KH * KW * PC;
 
-    int64_t *q = malloc(sizeof(int64_t) * (size_t)N * H * W * D);
     int64_t *padded = malloc(sizeof(int64_t) * (size_t)N * PH * PW * D);
     int64_t *rows = malloc(sizeof(int64_t) * (size_t)M * KH * KW * D);
     int32_t *acc = malloc(sizeof(int32_t) * (size_t)M * KN);
     int rc = -1;
-    if (q && padded && rows && acc) {
-        if (type < 2)
-            oracle_quantize_ternary(x, ths, N, H, W, C, q);
-        else
-            oracle_quantize_binary(x, ths, N, H, W, C, q);
-        oracle_pad(q, N, H, W, D, p1, p2, padded);
+    if (padded && rows && acc) {
+        oracle_pad(qx, N, H, W, D, p1, p2, padded);
         oracle_img2row(padded, N, PH, PW, D, KH, KW, s1, s2, rows);
         switch (type) {
         case 0: oracle_gemm_tnn(rows, qw, M, KN, K, acc); break;
         case 1: oracle_gemm_tbn(rows, qw, M, KN, K, acc); break;
         case 2: oracle_gemm_btn(rows, qw, btn, M, KN, K, acc); break;
-        default: oracle_gemm_bnn(rows, qw, M, KN, K, KH * KW * C, acc); break;
+        case 3: oracle_gemm_bnn(rows, qw, M, KN, K, KH * KW * C, acc); break;
+        case 4: oracle_gemm_drf(rows, qw, M, KN, K, acc); break;
+        default: oracle_gemm_rtn(rows, qw, M, KN, K, acc); break;
         }
 #pragma omp parallel for schedule(static)
         for (long i = 0; i < M * KN; i++) y[i] = (float)acc[i];
         rc = 0;
     }
-    free(q); free(padded); free(rows); free(acc);
+    free(padded); free(rows); free(acc);
+    return rc;
+}
+
+/*
+ * Whole Conv2d call (TAB_GEMM.cu:325-527): quantize the activation by type (ternary for
+ * 0/1, binary for 2/3; 419-426; for the CPU-only types, levels for 4 and ternary fields for
+ * 5), then the packed pipeline above with M=N*OH*OW, K=KH*KW*PC, NUM=KH*KW*C (509).  y holds
+ * the int result converted to fp32 at y[m*KN + kn], i.e. (n,oh,ow,kn) memory order
+ * (TAB_GEMM.cu:53,526).  Returns 0, or -1 on a bad type / empty output / allocation failure.
+ */
+int oracle_conv2d(const float *x, const int64_t *qw, const float *ths, const int32_t *btn,
+                  int type, int p1, int p2, int s1, int s2, int N, int H, int W, int C, int KN,
+                  int KH, int KW, float *y)
+{
+    if (type < 0 || type > 5) return -1;
+    const int PC = type == 5 ? (C + 31) / 32 : packed_channels(C);
+    const int D = (type < 2 || type == 4) ? PC * 2 : PC; /* activation words per pixel */
+    int64_t *q = malloc(sizeof(int64_t) * (size_t)N * H * W * D);
+    if (!q) return -1;
+    switch (type) {
+    case 0: case 1: oracle_quantize_ternary(x, ths, N, H, W, C, q); break;
+    case 2: case 3: oracle_quantize_binary(x, ths, N, H, W, C, q); break;
+    case 4: oracle_quantize_drf(x, ths, N, H, W, C, q); break;
+    default: oracle_quantize_rtn(x, ths, N, H, W, C, q); break;
+    }
+    const int rc = oracle_conv2d_packed(q, qw, btn, type, p1, p2, s1, s2, N, H, W, C, KN, KH, KW, y);
+    free(q);
     return rc;
 }

@@ -1,5 +1,5 @@
 """Writes tests/golden/ref_golden.npz: inputs and outputs of the reference's own CPU functions
-(TNN/TBN/BTN/BNNGEMM_baseline, TAB_CPU.cpp:242-328; Parallel_Img2Row_NHWCB_3x3,
+(TNN/TBN/BTN/BNN/DRF/RTNGEMM_baseline, TAB_CPU.cpp:242-383; Parallel_Img2Row_NHWCB_3x3,
 TAB_CPU.h:27-63; Parallel_Ternarize_NCHWB_to_NHWCB, TAB_CPU.cpp:20-124), run from
 oracle/_ref/libtab_ref.so, which oracle/Makefile compiles from /root/reference.
 
@@ -63,6 +63,14 @@ def main():
     out["bin_c128_x_chw"] = x
     out["bin_c128_dims"] = np.array([C, H, W, p1, p2], dtype=np.int64)
     out["bin_c128_q"] = oracle.ref_binarize_nchw(buf, p1, p2, 1, C, H, W)
+    # the CPU-only GEMMs (types 4 and 5), drawn last so that the vectors above keep their values
+    for t, (M, N, K) in zip((4, 5), [(18, 5, 6), (20, 8, 5)]):
+        planes = 2 if t == 4 else 1
+        a = rng.integers(-2**63, 2**63 - 1, size=(M, K, planes), dtype=np.int64, endpoint=True)
+        b = rng.integers(-2**63, 2**63 - 1, size=(N, K, planes), dtype=np.int64, endpoint=True)
+        out[f"gemm{t}_a"], out[f"gemm{t}_b"] = a, b
+        out[f"gemm{t}_mnk_num"] = np.array([M, N, K, 0], dtype=np.int64)
+        out[f"gemm{t}_y"] = oracle.ref_gemm(t, a, b, M, N, K)
     path = os.path.join(HERE, "ref_golden.npz")
     np.savez_compressed(path, **out)
     print("wrote", path, os.path.getsize(path), "bytes")

@@ -7,7 +7,7 @@ closed forms in numpy.
 import numpy as np
 import torch
 
-TYPE_NAMES = {0: "TNN", 1: "TBN", 2: "BTN", 3: "BNN"}
+TYPE_NAMES = {0: "TNN", 1: "TBN", 2: "BTN", 3: "BNN", 4: "DRF", 5: "RTN"}
 
 
 def act_bits(type):
@@ -81,6 +81,56 @@ def unpack(q, C, bitwidth):
     return (nz * (1 - 2 * sign)).astype(np.int8)
 
 
+# ---- the CPU-only types: DoReFa 2-bit levels (4) and RTN 2-bit fields (5) -------------------
+def brute_levels(x, ths):
+    """Levels 0..3 of the uniform quantizer with step ths[n]: bounds 0.5t, 1.5t, 2.5t in fp32."""
+    x = np.asarray(x, dtype=np.float32)
+    t = np.asarray(ths, dtype=np.float32)[: x.shape[0]].reshape((-1,) + (1,) * (x.ndim - 1))
+    with np.errstate(invalid="ignore"):
+        return ((x >= np.float32(0.5) * t).astype(np.int8) + (x >= np.float32(1.5) * t) + (x >= np.float32(2.5) * t)).astype(np.int8)
+
+
+def _pack_bits(bits, per_word):
+    """bits (..., L) of 0/1 -> uint64 words (..., ceil(L/per_word)), bit i of a word = element i."""
+    L = bits.shape[-1]
+    nw = (L + per_word - 1) // per_word
+    padded = np.zeros(bits.shape[:-1] + (nw * per_word,), dtype=np.uint64)
+    padded[..., :L] = bits
+    padded = padded.reshape(bits.shape[:-1] + (nw, per_word))
+    return (padded << np.arange(per_word, dtype=np.uint64)).sum(axis=-1, dtype=np.uint64)
+
+
+def pack_drf(levels):
+    """Levels (..., C) in 0..3 -> int64 (..., PC, 2): plane 0 the weight-2 bit, plane 1 the weight-1 bit."""
+    lv = np.asarray(levels).astype(np.uint64)
+    return np.stack([_pack_bits(lv >> np.uint64(1), 64), _pack_bits(lv & np.uint64(1), 64)], axis=-1).view(np.int64)
+
+
+def pack_rtn(values):
+    """Values (..., C) in {-1,0,+1} -> int64 (..., ceil(C/32)): field c%32 of word c//32, even bit =
+    nonzero, odd bit = sign."""
+    v = np.asarray(values)
+    fields = np.stack([(v != 0), (v < 0)], axis=-1).astype(np.uint64).reshape(v.shape[:-1] + (-1,))
+    return _pack_bits(fields, 64).view(np.int64)
+
+
+def unpack_drf(q, C):
+    """int64 (..., PC, 2) -> levels (..., C): 2 * plane 0 + plane 1, any bit pattern."""
+    q = np.ascontiguousarray(q).view(np.uint64)
+    bits = ((q[..., None] >> np.arange(64, dtype=np.uint64)) & np.uint64(1)).astype(np.int8)
+    hi = bits[..., 0, :].reshape(q.shape[:-2] + (-1,))[..., :C]
+    lo = bits[..., 1, :].reshape(q.shape[:-2] + (-1,))[..., :C]
+    return (2 * hi + lo).astype(np.int8)
+
+
+def unpack_rtn(q, C):
+    """int64 (..., PC32) -> values (..., C): nonzero bit * (1 - 2 * sign bit), any bit pattern."""
+    q = np.ascontiguousarray(q).view(np.uint64)
+    bits = ((q[..., None] >> np.arange(64, dtype=np.uint64)) & np.uint64(1)).astype(np.int8)
+    bits = bits.reshape(q.shape[:-1] + (-1, 2))[..., :C, :]
+    return (bits[..., 0] * (1 - 2 * bits[..., 1])).astype(np.int8)
+
+
 def torch_conv_reference(xq, wq, type, p1, p2, s1, s2, OH, OW):
     """Conv of dequantised tensors with torch: xq (N,H,W,C), wq (KN,KH,KW,C) in {-1,0,+1}.
     Padding value is 0 for ternary activations and +1 for binary ones (an all-zero packed
@@ -88,7 +138,7 @@ def torch_conv_reference(xq, wq, type, p1, p2, s1, s2, OH, OW):
     (n,oh,ow,kn) under an (N,KN,OH,OW) shape, like the reference's reshape."""
     x = torch.from_numpy(np.asarray(xq)).to(torch.float64).permute(0, 3, 1, 2)
     w = torch.from_numpy(np.asarray(wq)).to(torch.float64).permute(0, 3, 1, 2)
-    pad_value = 0.0 if act_bits(type) == 2 else 1.0
+    pad_value = 1.0 if type in (2, 3) else 0.0
     x = torch.nn.functional.pad(x, (p2, p2, p1, p1), value=pad_value)
     y = torch.nn.functional.conv2d(x, w, stride=(s1, s2))[:, :, :OH, :OW]
     N, KN = y.shape[0], y.shape[1]

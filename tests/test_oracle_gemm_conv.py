@@ -157,6 +157,6 @@ def test_conv2d_rejects_bad_arguments():
     x = np.zeros((1, 4, 4, 64), np.float32)
     qw = np.zeros((1, 3, 3, 1, 1), np.int64)
     with pytest.raises(ValueError):
-        oracle.conv2d(x, qw, [0.0], [0], 4, 1, 1, 1, 1, 1, 4, 4, 64, 1, 3, 3)
+        oracle.conv2d(x, qw, [0.0], [0], 6, 1, 1, 1, 1, 1, 4, 4, 64, 1, 3, 3)
     with pytest.raises(ValueError):
         oracle.conv2d(x, qw, [0.0], [0], 3, 0, 0, 1, 1, 1, 2, 2, 64, 1, 3, 3)  # empty output
