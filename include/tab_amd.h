@@ -15,6 +15,12 @@
  *        bits = 1: bit set <=> value -1                     TAB_GEMM.cu:196-197,238,321
  *   QW   the same layout with (N,H,W,C) = (KN,KH,KW,C)
  *   Y    fp32  [N*OH*OW][KN]  (labelled (N,KN,OH,OW) by the caller)   TAB_GEMM.cu:53,526
+ * and, for the two types that exist only in the reference's CPU file (TAB_CPU.cpp:332-383), the
+ * layouts their GEMMs read:
+ *   type 4 (DoReFa 2-bit)  int64 [N][H][W][PC][2], plane 0 = weight-2 bit, plane 1 = weight-1 bit of an
+ *        unsigned level 0..3, on both operands          TAB_CPU.cpp:345-354
+ *   type 5 (RTN)  int64 [N][H][W][ceil(C/32)], channel c -> word c/32, bit 2*(c%32) = nonzero marker,
+ *        bit 2*(c%32)+1 = sign marker, on both operands  TAB_CPU.cpp:364-379, 520-521
  */
 #ifndef TAB_AMD_H
 #define TAB_AMD_H
@@ -37,6 +43,8 @@ typedef enum tab_status {
 /* Conv types, TAB_GPU.cpp:27 ("0: TNN, 1, TBN, 2: BTN, 3: BNN"): first letter =
  * activation precision, second = weight precision. */
 enum { TAB_TNN = 0, TAB_TBN = 1, TAB_BTN = 2, TAB_BNN = 3 };
+/* The CPU path's two further types (TAB_CPU.cpp:577-584 / 603-610): DoReFa-Net 2-bit and RTN. */
+enum { TAB_DRF = 4, TAB_RTN = 5 };
 
 const char *tab_status_string(int status);
 const char *tab_last_error(void);
@@ -45,6 +53,11 @@ const char *tab_version(void);
 
 /* PC = ceil(C/64) (TAB_GEMM.cu:262-265). */
 int tab_packed_channels(int C);
+
+/* int64 words per pixel of the activation (operand 0) or per tap of the weight (operand 1) for conv
+ * type 0..5: planes * ceil(C/64), or ceil(C/32) for type 5 (TAB_GEMM.cu:367-379, TAB_CPU.cpp:520-521).
+ * 0 on bad arguments. */
+int tab_operand_words(int type, int operand, int C);
 
 /* Output extent (in + 2*pad - k + 1) / stride, integer division (TAB_GEMM.cu:354-357). */
 int tab_out_extent(int in, int pad, int k, int stride);
@@ -61,6 +74,20 @@ int tab_out_extent(int in, int pad, int k, int stride);
  */
 int tab_quantize(const float *dev_X, const float *dev_ths, int bitwidth, int N, int H, int W,
                  int C, int64_t *dev_QX, int32_t *dev_BTN, void *stream);
+
+/*
+ * Packers for conv types 4 and 5, activations and weights alike (weights as (N,H,W,C) = (KN,KH,KW,C)).
+ * The reference defines the word layouts through DRFGEMM_baseline / RTNGEMM_baseline
+ * (TAB_CPU.cpp:332-383) but ships no quantizer for them (TAB_Conv calls Parallel_Binarize_NCHW and
+ * Parallel_Ternarize_RTN, TAB_CPU.cpp:522,527, which no file defines), so the value rules are this
+ * library's:
+ *   type 4: level = (v >= 0.5t) + (v >= 1.5t) + (v >= 2.5t) with t = ths[n], the uniform 2-bit
+ *           quantizer with step t (each bound rounded to fp32; NaN -> 0)
+ *   type 5: the ternarizer's rule (v > t -> +1, else v < -t -> -1, TAB_GEMM.cu:184-192)
+ *   dev_QX  int64 [N*H*W*tab_operand_words(type, 0, C)], every element is written
+ */
+int tab_quantize_format(const float *dev_X, const float *dev_ths, int type, int N, int H, int W, int C,
+                        int64_t *dev_QX, void *stream);
 
 /*
  * Per-item threshold ths[n] = scale * mean(|X[n]|) over per_item consecutive fp32 values: the
@@ -97,6 +124,9 @@ size_t tab_conv2d_workspace_bytes(int type, int N, int H, int W, int C);
  *           passed this call
  * Padded taps read all-zero words: value 0 for ternary, +1 for binary activations
  * (TAB_CPU.cpp:39,155); BNN's constant is KH*KW*C (TAB_GEMM.cu:509).
+ * Types 4 and 5 (CPU-only in the reference, TAB_CPU.cpp:507-614) are accepted too: X goes through
+ * tab_quantize_format, dev_QW holds the same format, zero words are the value 0, and Y is
+ * DRFGEMM_baseline's / RTNGEMM_baseline's integer as fp32.  Type 4 needs 9 * 64 * K words < 2^24.
  */
 int tab_conv2d(const float *dev_X, const int64_t *dev_QW, const float *dev_ths,
                const int32_t *dev_btn, int type, int padding1, int padding2, int stride1,
@@ -107,7 +137,8 @@ int tab_conv2d(const float *dev_X, const int64_t *dev_QW, const float *dev_ths,
  * The second half of tab_conv2d on an activation that is already packed (the output of
  * tab_quantize with bitwidth 2 for TNN/TBN, 1 for BTN/BNN): zero padding, im2row and the
  * popcount GEMM (PadKernel + Img2RowKernel + GEMMWithCuda, TAB_GEMM.cuh:22-115) fused in
- * one kernel.  dev_QX int64 [N*H*W*PC*abits]; other arguments as in tab_conv2d.
+ * one kernel.  dev_QX int64 [N*H*W*PC*abits]; other arguments as in tab_conv2d.  Types 4 and 5:
+ * dev_QX int64 [N*H*W*tab_operand_words(type, 0, C)] from tab_quantize_format.
  */
 int tab_conv2d_packed(const int64_t *dev_QX, const int64_t *dev_QW, const int32_t *dev_btn,
                       int type, int padding1, int padding2, int stride1, int stride2, int N,
@@ -122,6 +153,7 @@ int tab_conv2d_packed(const int64_t *dev_QX, const int64_t *dev_QW, const int32_
  * reference has no counterpart (every TAB_Conv2d returns fp32 and the caller re-quantizes).
  *   dev_out_ths fp32 [>=N]: threshold for the outputs of image n
  *   dev_QY      int64 [N*OH*OW*ceil(KN/64)*out_bitwidth], every element is written
+ * Types 0..3 only.
  */
 int tab_conv2d_packed_out(const int64_t *dev_QX, const int64_t *dev_QW, const int32_t *dev_btn,
                           int type, int padding1, int padding2, int stride1, int stride2, int N,
@@ -138,6 +170,7 @@ int tab_conv2d_packed_out(const int64_t *dev_QX, const int64_t *dev_QW, const in
  *                      four waves, 4: 256x64, 5: 256x128, 6: 128x256; -1: picked from the shape
  *   TAB_CONV_POPCOUNT  the reference's xor/and + popcount formulation on the vector ALU;
  *                      tile 0: big, 1: medium, 2: small; -1: picked from the shape
+ *                      (types 4 and 5 exist on the matrix cores only and ignore this choice)
  */
 enum { TAB_CONV_AUTO = 0, TAB_CONV_MATRIX = 1, TAB_CONV_POPCOUNT = 2 };
 int tab_set_conv_kernel(int kernel, int tile);

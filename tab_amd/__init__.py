@@ -15,6 +15,7 @@ _lib = _capi.load()
 TabError = _capi.TabError
 
 TNN, TBN, BTN, BNN = 0, 1, 2, 3
+DRF, RTN = 4, 5  # the types of the reference's CPU path only (TAB_CPU.cpp:332-383)
 
 
 def version():
@@ -44,6 +45,11 @@ def _stream():
 
 def packed_channels(C):
     return _lib.tab_packed_channels(int(C))
+
+
+def operand_words(type, operand, C):
+    """int64 words per pixel of the activation (operand 0) or per tap of the weight (operand 1)."""
+    return _lib.tab_operand_words(int(type), int(operand), int(C))
 
 
 def out_shape(H, W, KH, KW, pad1, pad2, stride1, stride2):
@@ -79,6 +85,35 @@ def Quantize(X, thresholds, bitwidth, N, H, W, C):
     return [QX, BTN]
 
 
+def QuantizeFormat(X, thresholds, type, N, H, W, C):
+    """Packer of conv types 4 (DoReFa 2-bit levels; QX int64 (N,H,W,PC,2), plane 0 = weight-2 bit)
+    and 5 (RTN 2-bit fields; QX int64 (N,H,W,ceil(C/32))), for activations and weights alike.  The
+    layouts are the ones DRFGEMM_baseline / RTNGEMM_baseline read (TAB_CPU.cpp:332-383); the
+    reference has no quantizer for them, the value rules (uniform step thresholds[n]; the
+    ternarizer's compares) are this library's."""
+    _check_input(X, "X")
+    _check_input(thresholds, "thresholds")
+    _check_dtype(X, torch.float32, "X")
+    _check_dtype(thresholds, torch.float32, "thresholds")
+    type, N, H, W, C = int(type), int(N), int(H), int(W), int(C)
+    if type not in (DRF, RTN):
+        raise RuntimeError(f"type must be 4 (DRF) or 5 (RTN), got {type}")
+    if min(N, H, W, C) < 1:
+        raise RuntimeError("N, H, W, C must be positive")
+    if X.numel() != N * H * W * C:
+        raise RuntimeError(f"X has {X.numel()} elements, expected N*H*W*C = {N * H * W * C}")
+    if thresholds.numel() < N:
+        raise RuntimeError(f"thresholds has {thresholds.numel()} elements, expected at least N = {N}")
+    if thresholds.device != X.device:
+        raise RuntimeError("X and thresholds must be on the same device")
+    shape = (N, H, W, packed_channels(C), 2) if type == DRF else (N, H, W, (C + 31) // 32)
+    with torch.cuda.device(X.device):
+        QX = torch.empty(shape, dtype=torch.int64, device=X.device)
+        _capi.check(_lib, _lib.tab_quantize_format(X.data_ptr(), thresholds.data_ptr(), type, N, H, W, C,
+                                                   QX.data_ptr(), _stream()))
+    return QX
+
+
 def Threshold(X, N, scale=0.7):
     """ths[n] = scale * mean(|X[n]|) per item (image or filter), fp32 (N,), computed on the
     device in one pass: the threshold rule the reference leaves to the caller (README.md:45).
@@ -99,14 +134,13 @@ def Threshold(X, N, scale=0.7):
 
 
 def _conv_checks(QW, btn, type, N, H, W, C, KN, KH, KW, pad1, pad2, stride1, stride2):
-    if type not in (0, 1, 2, 3):
-        raise RuntimeError(f"type must be 0 (TNN), 1 (TBN), 2 (BTN) or 3 (BNN), got {type}")
+    if type not in (0, 1, 2, 3, 4, 5):
+        raise RuntimeError(f"type must be 0 (TNN), 1 (TBN), 2 (BTN), 3 (BNN), 4 (DRF) or 5 (RTN), got {type}")
     if min(N, H, W, C, KN, KH, KW) < 1 or min(pad1, pad2) < 0 or min(stride1, stride2) < 1:
         raise RuntimeError("sizes must be positive, padding >= 0 and stride >= 1")
-    wbits = 2 if type in (0, 2) else 1
-    need = KN * KH * KW * packed_channels(C) * wbits
+    need = KN * KH * KW * operand_words(type, 1, C)
     if QW.numel() != need:
-        raise RuntimeError(f"QW has {QW.numel()} words, type {type} expects KN*KH*KW*PC*{wbits} = {need}")
+        raise RuntimeError(f"QW has {QW.numel()} words, type {type} expects KN*KH*KW*{operand_words(type, 1, C)} = {need}")
     if type == 2 and btn.numel() < KN:
         raise RuntimeError(f"btn has {btn.numel()} elements, expected at least KN = {KN}")
     OH, OW = out_shape(H, W, KH, KW, pad1, pad2, stride1, stride2)
@@ -116,8 +150,8 @@ def _conv_checks(QW, btn, type, N, H, W, C, KN, KH, KW, pad1, pad2, stride1, str
 
 
 def Conv2d(X, QW, thresholds, btn, type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW):
-    """Quantize the NHWC fp32 activation on the fly (ternary for types 0/1, binary for 2/3)
-    and convolve it with the packed weights by XOR/AND + popcount.  Returns fp32 shaped
+    """Quantize the NHWC fp32 activation on the fly (ternary for types 0/1, binary for 2/3; types 4
+    and 5 of the CPU path through QuantizeFormat) and convolve it with the packed weights.  Returns fp32 shaped
     (N,KN,OH,OW) whose memory is ordered (n,oh,ow,kn), exactly as the reference's reshape
     of its GEMM result (TAB_GPU.cpp:34-42, TAB_GEMM.cu:325-527)."""
     for t, name in ((X, "X"), (QW, "QW"), (thresholds, "thresholds"), (btn, "btn")):
@@ -148,7 +182,8 @@ def Conv2d(X, QW, thresholds, btn, type, padding1, padding2, stride1, stride2, N
 
 def Conv2dPacked(QX, QW, btn, type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW):
     """Conv2d on an activation already packed by Quantize (bitwidth 2 for types 0/1,
-    1 for types 2/3): the pad + im2row + GEMM stages of TAB_GEMM.cu:447-509 only."""
+    1 for types 2/3) or by QuantizeFormat (types 4/5): the pad + im2row + GEMM stages of
+    TAB_GEMM.cu:447-509 only."""
     for t, name in ((QX, "QX"), (QW, "QW"), (btn, "btn")):
         _check_input(t, name)
     _check_dtype(QX, torch.int64, "QX")
@@ -157,9 +192,8 @@ def Conv2dPacked(QX, QW, btn, type, padding1, padding2, stride1, stride2, N, H, 
     (type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW) = (
         int(v) for v in (type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW))
     OH, OW = _conv_checks(QW, btn, type, N, H, W, C, KN, KH, KW, padding1, padding2, stride1, stride2)
-    abits = 2 if type < 2 else 1
-    if QX.numel() != N * H * W * packed_channels(C) * abits:
-        raise RuntimeError(f"QX has {QX.numel()} words, type {type} expects N*H*W*PC*{abits}")
+    if QX.numel() != N * H * W * operand_words(type, 0, C):
+        raise RuntimeError(f"QX has {QX.numel()} words, type {type} expects N*H*W*{operand_words(type, 0, C)}")
     with torch.cuda.device(QX.device):
         Y = torch.empty((N, KN, OH, OW), dtype=torch.float32, device=QX.device)
         _capi.check(_lib, _lib.tab_conv2d_packed(QX.data_ptr(), QW.data_ptr(), btn.data_ptr(), type,
@@ -183,6 +217,8 @@ def Conv2dPackedOut(QX, QW, btn, type, padding1, padding2, stride1, stride2, N, 
     _check_dtype(out_thresholds, torch.float32, "out_thresholds")
     (type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW, out_bitwidth) = (
         int(v) for v in (type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW, out_bitwidth))
+    if type not in (0, 1, 2, 3):
+        raise RuntimeError(f"packed output exists for types 0..3 only, got {type}")
     OH, OW = _conv_checks(QW, btn, type, N, H, W, C, KN, KH, KW, padding1, padding2, stride1, stride2)
     abits = 2 if type < 2 else 1
     if QX.numel() != N * H * W * packed_channels(C) * abits:
@@ -212,6 +248,6 @@ def set_conv_kernel(kernel=CONV_AUTO, tile=-1):
 TAB_Quantize = Quantize
 TAB_Conv2d = Conv2d
 
-__all__ = ["Quantize", "Conv2d", "Conv2dPacked", "Conv2dPackedOut", "Threshold", "TAB_Quantize", "TAB_Conv2d", "TabError",
+__all__ = ["Quantize", "QuantizeFormat", "Conv2d", "Conv2dPacked", "Conv2dPackedOut", "Threshold", "TAB_Quantize", "TAB_Conv2d", "TabError",
            "packed_channels", "out_shape", "version", "TNN", "TBN", "BTN", "BNN", "set_conv_kernel",
            "CONV_AUTO", "CONV_MATRIX", "CONV_POPCOUNT"]

@@ -16,8 +16,10 @@ SIGNATURES = {
     "tab_last_error": (ctypes.c_char_p, []),
     "tab_version": (ctypes.c_char_p, []),
     "tab_packed_channels": (_int, [_int]),
+    "tab_operand_words": (_int, [_int] * 3),
     "tab_out_extent": (_int, [_int] * 4),
     "tab_quantize": (_int, [_vp, _vp, _int, _int, _int, _int, _int, _vp, _vp, _vp]),
+    "tab_quantize_format": (_int, [_vp, _vp, _int, _int, _int, _int, _int, _vp, _vp]),
     "tab_threshold_workspace_bytes": (_sz, [_int, ctypes.c_long]),
     "tab_threshold": (_int, [_vp, _int, ctypes.c_long, ctypes.c_float, _vp, _vp, _sz, _vp]),
     "tab_conv2d_workspace_bytes": (_sz, [_int] * 5),

@@ -35,23 +35,27 @@ struct ConvShape {
 int check_conv(int type, int p1, int p2, int s1, int s2, int N, int H, int W, int C, int KN,
                int KH, int KW, ConvShape *s)
 {
-    if (type < 0 || type > 3) return fail(TAB_ERR_BAD_ARGUMENT, "type must be 0 (TNN), 1 (TBN), 2 (BTN) or 3 (BNN), got %d", type);
+    if (type < 0 || type > 5)
+        return fail(TAB_ERR_BAD_ARGUMENT, "type must be 0 (TNN), 1 (TBN), 2 (BTN), 3 (BNN), 4 (DRF) or 5 (RTN), got %d", type);
     if (N < 1 || H < 1 || W < 1 || C < 1 || KN < 1 || KH < 1 || KW < 1)
         return fail(TAB_ERR_BAD_ARGUMENT, "N, H, W, C, KN, KH, KW must be positive");
     if (p1 < 0 || p2 < 0 || s1 < 1 || s2 < 1)
         return fail(TAB_ERR_BAD_ARGUMENT, "padding must be >= 0 and stride >= 1");
-    s->PC = tab_packed_channels(C);
+    s->PC = type == TAB_RTN ? (C + 31) / 32 : tab_packed_channels(C);
     s->OH = tab_out_extent(H, p1, KH, s1);
     s->OW = tab_out_extent(W, p2, KW, s2);
     if (s->OH < 1 || s->OW < 1)
         return fail(TAB_ERR_BAD_SHAPE, "empty output: OH=%d OW=%d", s->OH, s->OW);
-    s->abits = (type < 2) ? 2 : 1;
-    s->wbits = (type == 0 || type == 2) ? 2 : 1;
+    s->abits = (type < 2 || type == TAB_DRF) ? 2 : 1;  // planes per word position, TAB_CPU.cpp:345-354 for type 4
+    s->wbits = (type == 0 || type == 2 || type == TAB_DRF) ? 2 : 1;
     s->M = (long)N * s->OH * s->OW;
     s->G = (long)KH * KW * s->PC;
     if (s->M > kMaxIndex - 512 || s->G >= 65536 || s->PC >= 65536 || KW >= 65536 ||
         (long)N * H * W > kMaxIndex || (long)H * W * s->PC * 2 > kMaxIndex)
         return fail(TAB_ERR_BAD_SHAPE, "problem too large for 32-bit row indices (M=%ld, K words=%ld)", s->M, s->G);
+    // type 4 multiplies levels up to 3: 9 * 64 * G has to stay below 2^24 for the fp32 accumulators
+    if (type == TAB_DRF && s->G * 64 * 9 >= (1L << 24))
+        return fail(TAB_ERR_BAD_SHAPE, "K of %ld words is too long for exact accumulation of type 4", s->G);
     // a workgroup addresses the images its (at most 256) output pixels touch with 32-bit byte offsets
     const long image_bytes = (long)H * W * s->PC * s->abits * 8;
     if (image_bytes * (256 / ((long)s->OH * s->OW) + 2) > 0xffffffffL)
@@ -133,11 +137,30 @@ int tab_threshold(const float *dev_X, int N, long per_item, float scale, float *
     return TAB_OK;
 }
 
+int tab_operand_words(int type, int operand, int C)
+{
+    if (type < 0 || type > 5 || operand < 0 || operand > 1 || C < 1) return 0;
+    if (type == TAB_RTN) return (C + 31) / 32;
+    const bool two_planes = type == TAB_DRF || (operand == 0 ? type < 2 : (type == 0 || type == 2));
+    return tab_packed_channels(C) * (two_planes ? 2 : 1);
+}
+
 size_t tab_conv2d_workspace_bytes(int type, int N, int H, int W, int C)
 {
-    if (type < 0 || type > 3 || N < 1 || H < 1 || W < 1 || C < 1) return 0;
-    const size_t abits = (type < 2) ? 2 : 1;
-    return (size_t)N * H * W * tab_packed_channels(C) * abits * sizeof(int64_t);
+    if (type < 0 || type > 5 || N < 1 || H < 1 || W < 1 || C < 1) return 0;
+    return (size_t)N * H * W * tab_operand_words(type, 0, C) * sizeof(int64_t);
+}
+
+int tab_quantize_format(const float *dev_X, const float *dev_ths, int type, int N, int H, int W, int C,
+                        int64_t *dev_QX, void *stream)
+{
+    if (type != TAB_DRF && type != TAB_RTN) return fail(TAB_ERR_BAD_ARGUMENT, "type must be 4 (DRF) or 5 (RTN), got %d", type);
+    if (N < 1 || H < 1 || W < 1 || C < 1) return fail(TAB_ERR_BAD_ARGUMENT, "N, H, W, C must be positive");
+    if (!dev_X || !dev_ths || !dev_QX) return fail(TAB_ERR_BAD_ARGUMENT, "null device pointer");
+    hipError_t e = tab::launch_quantize_format(dev_X, dev_ths, type, (long)H * W, N, C, reinterpret_cast<uint64_t *>(dev_QX),
+                                               static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return device_fail(e, "quantize launch");
+    return TAB_OK;
 }
 
 /* Shared body of the packed-activation entry points: Y as fp32 (dev_Y) or thresholded and packed (dev_QY). */
@@ -153,6 +176,7 @@ static int conv_packed(const int64_t *dev_QX, const int64_t *dev_QW, const int32
     if (((uintptr_t)dev_QX % (8 * s.abits)) || ((uintptr_t)dev_QW % (8 * s.wbits)) || ((uintptr_t)dev_Y % 16))
         return fail(TAB_ERR_BAD_ARGUMENT, "QX/QW must be aligned to a whole packed element and Y to 16 bytes");
     if (dev_QY) {
+        if (type > 3) return fail(TAB_ERR_BAD_ARGUMENT, "packed output exists for types 0..3 only, got %d", type);
         if (out_bitwidth != 1 && out_bitwidth != 2)
             return fail(TAB_ERR_BAD_ARGUMENT, "out_bitwidth must be 1 or 2, got %d", out_bitwidth);
         if (!dev_out_ths) return fail(TAB_ERR_BAD_ARGUMENT, "null device pointer");
@@ -216,6 +240,13 @@ int tab_conv2d(const float *dev_X, const int64_t *dev_QW, const float *dev_ths,
     // A 1x1 convolution with stride and no padding reads one pixel in stride1*stride2: quantize only
     // those, into a compact activation, and convolve it with stride 1 (same outputs, a fraction of
     // the reads of X).
+    if (type > 3) {  // the CPU-only types: their own packers, then the same fused kernel
+        hipError_t e = tab::launch_quantize_format(dev_X, dev_ths, type, (long)H * W, N, C, reinterpret_cast<uint64_t *>(workspace),
+                                                   static_cast<hipStream_t>(stream));
+        if (e != hipSuccess) return device_fail(e, "quantize launch");
+        return tab_conv2d_packed(reinterpret_cast<const int64_t *>(workspace), dev_QW, dev_btn, type, padding1, padding2, stride1,
+                                 stride2, N, H, W, C, KN, KH, KW, dev_Y, stream);
+    }
     if (KH == 1 && KW == 1 && padding1 == 0 && padding2 == 0 && (stride1 > 1 || stride2 > 1) && N * (long)s.OH < 65536 &&
         tab::quantize_strided_supported(dev_X, H, W, C, s.OH, s.OW)) {
         hipError_t e = tab::launch_quantize_strided(dev_X, dev_ths, s.abits, N, H, W, C, s.OH, s.OW, stride1, stride2,

@@ -29,7 +29,7 @@ __device__ __forceinline__ uint32_t fastdiv(uint32_t x, FastDiv f)
 
 // Arguments of the fused pad + im2row + popcount-GEMM kernel.
 struct ConvArgs {
-    const uint64_t *qx;  // packed activation [N][H][W][PC][APL]
+    const uint64_t *qx;  // packed activation [N][H][W][PC][APL]; PC = words per pixel and plane
     const uint64_t *qw;  // packed weight     [KN][KH][KW][PC][BPL]
     const int32_t *btn;  // [KN] (BTN only)
     float *y;            // [M][KN]
@@ -56,14 +56,21 @@ hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream);
 // Matrix-core (FP4 MFMA) variant; shape picks the workgroup tile.  conv_mfma_exact() says whether K is
 // short enough for its fp32 accumulators to hold every partial sum exactly.
 bool conv_mfma_exact(const ConvArgs &args);
+bool conv_mfma_exact_levels(const ConvArgs &args);  // the same for type 4, whose products reach 9
 int conv_mfma_shape(int type, const ConvArgs &args);
 hipError_t launch_conv_mfma(int type, const ConvArgs &args, int shape, hipStream_t stream);
 hipError_t launch_conv_mfma_tnn(const ConvArgs &args, int shape, hipStream_t stream);
 hipError_t launch_conv_mfma_tbn(const ConvArgs &args, int shape, hipStream_t stream);
 hipError_t launch_conv_mfma_btn(const ConvArgs &args, int shape, hipStream_t stream);
 hipError_t launch_conv_mfma_bnn(const ConvArgs &args, int shape, hipStream_t stream);
+hipError_t launch_conv_mfma_drf(const ConvArgs &args, int shape, hipStream_t stream);
+hipError_t launch_conv_mfma_rtn(const ConvArgs &args, int shape, hipStream_t stream);
 hipError_t launch_quantize(const float *x, const float *ths, int bitwidth, long pixels_per_item,
                            long items, int C, uint64_t *qx, int32_t *btn, hipStream_t stream);
+
+// Packers of the CPU-only conv types: format 4 = DoReFa 2-bit levels, 5 = RTN fields.
+hipError_t launch_quantize_format(const float *x, const float *ths, int format, long pixels_per_item, long items, int C,
+                                  uint64_t *qx, hipStream_t stream);
 
 // Quantize only the pixels (oh*s1, ow*s2) of every image into a compact [N][OH][OW][PC] activation
 // (what a 1x1 convolution with stride and no padding reads).

@@ -331,7 +331,10 @@ void force_conv_tile(int tm, int ng)
     g_force_ng = ng;
 }
 
+// fp32 accumulators hold integers up to 2^24 exactly; a product is at most 1 (9 for the 2-bit levels of
+// type 4, see conv_mfma_exact_levels) and there are 64 per word
 bool conv_mfma_exact(const ConvArgs &a) { return (long)a.G * 64 <= (1L << 22); }
+bool conv_mfma_exact_levels(const ConvArgs &a) { return (long)a.G * 64 * 9 < (1L << 24); }
 
 hipError_t launch_conv_mfma(int type, const ConvArgs &args, int shape, hipStream_t stream)
 {
@@ -341,6 +344,8 @@ hipError_t launch_conv_mfma(int type, const ConvArgs &args, int shape, hipStream
     case 1: return launch_conv_mfma_tbn(args, shape, stream);
     case 2: return launch_conv_mfma_btn(args, shape, stream);
     case 3: return launch_conv_mfma_bnn(args, shape, stream);
+    case 4: return conv_mfma_exact_levels(args) ? launch_conv_mfma_drf(args, shape, stream) : hipErrorInvalidValue;
+    case 5: return launch_conv_mfma_rtn(args, shape, stream);
     default: return hipErrorInvalidValue;
     }
 }
@@ -349,8 +354,10 @@ hipError_t launch_conv_mfma(int type, const ConvArgs &args, int shape, hipStream
 // N = 8 .. 256: the 128-row tiles win as soon as there is about one of them per CU (the 128x128 one
 // with short K they need about four per CU); below roughly 200 workgroups of 64x64 the launch is
 // latency-bound and the k-split 32x32 shape wins.
-int conv_mfma_shape(int type, const ConvArgs &a)
+int conv_mfma_shape(int conv_type, const ConvArgs &a)
 {
+    // the CPU-only types follow the type with the same planes: 4 like TNN, 5 like BNN
+    const int type = conv_type == 4 ? 0 : (conv_type == 5 ? 3 : conv_type);
     auto tiles = [&](int bm, int bn) { return (long)((a.M + bm - 1) / bm) * ((a.KN + bn - 1) / bn); };
     const long enough = a.G >= 36 ? 300 : 1024;  // short K: the per-tile prologue and epilogue weigh more
     // eight tiles per wave share each expanded operand between more MFMAs (the dearer operand gets the
@@ -383,6 +390,8 @@ hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream)
     // default path: matrix cores; the popcount kernel takes over when K is too long for exact fp32
     // accumulation (and when a benchmark forces one of its tiles)
     if (g_force_tm == 0 && conv_mfma_exact(args)) return launch_conv_mfma(type, args, conv_mfma_shape(type, args), stream);
+    // types 4 and 5 exist on the matrix cores only
+    if (type > 3) return launch_conv_mfma(type, args, conv_mfma_shape(type, args), stream);
     switch (type) {
     case 0: return launch_type<0>(args, stream);
     case 1: return launch_type<1>(args, stream);

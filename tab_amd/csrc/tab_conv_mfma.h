@@ -81,6 +81,43 @@ __device__ __forceinline__ i32x8 expand_ternary(uint32_t s, uint32_t z, const Ex
     return r;
 }
 
+// Type 4 (TAB_CPU.cpp:332-358): planes (hi, lo) of a level 0..3 on both sides; E2M1 holds 1 = 0010,
+// 2 = 0100 and 3 = 0101 exactly, so exponent bit 1 = hi, exponent bit 0 = lo & ~hi, mantissa = hi & lo,
+// and the products (at most 9) and their sums stay exact integers.
+__device__ __forceinline__ i32x8 expand_levels(uint32_t hi, uint32_t lo)
+{
+    const uint32_t one = lo & ~hi, three = hi & lo;
+    i32x8 r = {0, 0, 0, 0, 0, 0, 0, 0};
+    r[0] = (int)(((hi & kBit0) << 2) | ((one & kBit0) << 1) | (three & kBit0));
+    r[1] = (int)(((hi & kBit1) << 1) | (one & kBit1) | ((three & kBit1) >> 1));
+    r[2] = (int)((hi & kBit2) | ((one & kBit2) >> 1) | ((three & kBit2) >> 2));
+    r[3] = (int)(((hi & kBit3) >> 1) | ((one & kBit3) >> 2) | ((three & kBit3) >> 3));
+    return r;
+}
+
+// Type 5 (TAB_CPU.cpp:362-383): a 32-bit slice holds 16 fields (even bit = nonzero, odd bit = sign).
+// The fields at even positions of the slice fill operand dword 0, those at odd positions dword 1,
+// each as the nibble (sign, 0, nonzero, 0) = +-1 or +-0; a slice is 16 of the 32 elements a lane can
+// feed, the other operand dwords stay zero.
+__device__ __forceinline__ i32x8 expand_fields(uint32_t w)
+{
+    i32x8 r = {0, 0, 0, 0, 0, 0, 0, 0};
+    r[0] = (int)(((w << 1) & kBit1) | ((w << 2) & kBit3));
+    r[1] = (int)(((w >> 1) & kBit1) | (w & kBit3));
+    return r;
+}
+
+// The FP4 operand of one 32-bit slice: SIDE 0 = activation, 1 = weight; p0, p1 = the slice of plane 0
+// and of the last plane (the same word for one-plane operands).
+template <int TYPE, int SIDE>
+__device__ __forceinline__ i32x8 expand_operand(uint32_t p0, uint32_t p1, const ExpandConsts &c)
+{
+    if (TYPE == 4) return expand_levels(p0, p1);
+    if (TYPE == 5) return expand_fields(p0);
+    constexpr int PL = SIDE ? Planes<TYPE>::B : Planes<TYPE>::A;
+    return PL == 2 ? expand_ternary<SIDE>(p0, p1, c) : expand_binary<SIDE>(p0, c);
+}
+
 // waves_per_eu: the shapes with four MFMA tiles per wave are capped at 128 registers, i.e. four
 // workgroups per CU (the 128x128 shape otherwise takes 136-152, 64 of them accumulators, and runs
 // three, measured 3-7 % slower); 256-row tiles need the state of more staged rows and get 168
@@ -167,10 +204,10 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
             i32x8 af[TM], bf[TN];
 #pragma unroll
             for (int mt = 0; mt < TM; mt++)
-                af[mt] = (APL == 2) ? expand_ternary<0>(a_w[w][0][mt], a_w[w][APL - 1][mt], consts) : expand_binary<0>(a_w[w][0][mt], consts);
+                af[mt] = expand_operand<TYPE, 0>(a_w[w][0][mt], a_w[w][APL - 1][mt], consts);
 #pragma unroll
             for (int nt = 0; nt < TN; nt++) {
-                bf[nt] = (BPL == 2) ? expand_ternary<1>(b_w[w][0][nt], b_w[w][BPL - 1][nt], consts) : expand_binary<1>(b_w[w][0][nt], consts);
+                bf[nt] = expand_operand<TYPE, 1>(b_w[w][0][nt], b_w[w][BPL - 1][nt], consts);
                 if (TYPE == 2) b_nonzero[nt] += __builtin_popcount(b_w[w][BPL - 1][nt]);
             }
 #pragma unroll

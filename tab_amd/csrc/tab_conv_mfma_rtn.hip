@@ -1,0 +1,10 @@
+// RTN (type 5) instantiations of the matrix-core conv kernel (one translation unit per type so they
+// compile in parallel).
+#include "tab_conv_mfma.h"
+
+namespace tab {
+hipError_t launch_conv_mfma_rtn(const ConvArgs &args, int shape, hipStream_t stream)
+{
+    return launch_mfma_type<5>(args, shape, stream);
+}
+}  // namespace tab

@@ -17,9 +17,11 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
+// Types 4 (DoReFa 2-bit levels, two planes on both sides) and 5 (RTN, 2-bit fields interleaved in one
+// plane on both sides) are the CPU-only ones of the reference (TAB_CPU.cpp:332-383).
 template <int TYPE> struct Planes {
-    static constexpr int A = (TYPE == 0 || TYPE == 1) ? 2 : 1;  // activation planes (TAB_GEMM.cu:367-372)
-    static constexpr int B = (TYPE == 0 || TYPE == 2) ? 2 : 1;  // weight planes (TAB_GEMM.cu:374-379)
+    static constexpr int A = (TYPE == 0 || TYPE == 1 || TYPE == 4) ? 2 : 1;  // activation planes (TAB_GEMM.cu:367-372)
+    static constexpr int B = (TYPE == 0 || TYPE == 2 || TYPE == 4) ? 2 : 1;  // weight planes (TAB_GEMM.cu:374-379)
 };
 
 // One packed word (all planes) of one row of an operand, held in registers between the

@@ -202,6 +202,48 @@ __global__ __launch_bounds__(kThreads) void quantize_ballot(const float *__restr
     }
 }
 
+// Packers of the two CPU-only conv types, whose word layouts follow from the reference's GEMMs (it has
+// no quantizer for them: TAB_Conv calls Parallel_Binarize_NCHW and Parallel_Ternarize_RTN,
+// TAB_CPU.cpp:522,527, which no file defines).  One wave per output word, ballots as above.
+// FORMAT 4, DoReFa 2-bit (DRFGEMM_baseline, TAB_CPU.cpp:345-354): [pixel][ceil(C/64)][2], plane 0 the
+//   weight-2 bit and plane 1 the weight-1 bit of level = (v >= 0.5t) + (v >= 1.5t) + (v >= 2.5t).
+// FORMAT 5, RTN (RTNGEMM_baseline, TAB_CPU.cpp:364-379; 32 channels per word, 520-521):
+//   [pixel][ceil(C/32)], channel c in word c/32 as the field (bit 2*(c%32) = nonzero, bit 2*(c%32)+1 =
+//   sign) of the ternarizer's value; lane j of the wave tests channel j/2 for bit j.
+template <int FORMAT>
+__global__ __launch_bounds__(kThreads) void quantize_ballot_format(const float *__restrict__ x, const float *__restrict__ ths,
+                                                                   uint64_t *__restrict__ q, long pixels,
+                                                                   long pixels_per_item, int C, int PC)
+{
+    const int lane = threadIdx.x & 63;
+    const long nwaves = (long)gridDim.x * kWavesPerBlock;
+    const long units = pixels * PC;
+    for (long unit = (long)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6); unit < units; unit += nwaves) {
+        const long pixel = unit / PC;
+        const int word = (int)(unit - pixel * PC);
+        const float t = ths[pixel / pixels_per_item];
+        if (FORMAT == 4) {
+            const int c = word * kWordBits + lane;
+            const bool live = c < C;
+            const float v = live ? x[pixel * C + c] : 0.f;
+            const int level = live ? (int)(v >= 0.5f * t) + (int)(v >= 1.5f * t) + (int)(v >= 2.5f * t) : 0;
+            const uint64_t hi = __ballot(level >> 1), lo = __ballot(level & 1);
+            if (lane == 0) {
+                q[unit * 2 + 0] = hi;
+                q[unit * 2 + 1] = lo;
+            }
+        } else {
+            const int c = word * 32 + (lane >> 1);
+            const bool live = c < C;
+            const float v = live ? x[pixel * C + c] : 0.f;
+            const bool pos = live && (v > t);
+            const bool neg = live && !pos && (v < -t);
+            const uint64_t fields = __ballot((lane & 1) ? neg : (pos || neg));
+            if (lane == 0) q[unit] = fields;
+        }
+    }
+}
+
 __global__ void fill_zero_i32(int32_t *p, long n)
 {
     const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -354,6 +396,24 @@ hipError_t launch_quantize(const float *x, const float *ths, int bitwidth, long 
         btn_popcount<<<dim3((unsigned)(items * splits)), dim3(kThreads), 0, stream>>>(
             reinterpret_cast<const ulonglong2 *>(qx), btn, words_per_item, splits);
     }
+    return hipGetLastError();
+}
+
+hipError_t launch_quantize_format(const float *x, const float *ths, int format, long pixels_per_item, long items, int C,
+                                  uint64_t *qx, hipStream_t stream)
+{
+    const int PC = format == 5 ? (C + 31) / 32 : (C + kWordBits - 1) / kWordBits;
+    const long pixels = items * pixels_per_item;
+    const long units = pixels * PC;
+    long blocks = (units + kWavesPerBlock - 1) / kWavesPerBlock;
+    if (blocks > 256 * 32) blocks = 256 * 32;  // grid-stride beyond 32 blocks per CU
+    const dim3 grid((unsigned)blocks), block(kThreads);
+    if (format == 4)
+        quantize_ballot_format<4><<<grid, block, 0, stream>>>(x, ths, qx, pixels, pixels_per_item, C, PC);
+    else if (format == 5)
+        quantize_ballot_format<5><<<grid, block, 0, stream>>>(x, ths, qx, pixels, pixels_per_item, C, PC);
+    else
+        return hipErrorInvalidValue;
     return hipGetLastError();
 }
 

@@ -42,7 +42,13 @@ def test_host_only_entry_points():
     # activation scratch: N*H*W*PC*abits int64 words
     assert lib.tab_conv2d_workspace_bytes(0, 2, 5, 5, 70) == 2 * 5 * 5 * 2 * 2 * 8
     assert lib.tab_conv2d_workspace_bytes(3, 2, 5, 5, 70) == 2 * 5 * 5 * 2 * 1 * 8
-    assert lib.tab_conv2d_workspace_bytes(4, 2, 5, 5, 70) == 0
+    # the CPU-only types: two planes of ceil(C/64) words (4), one plane of ceil(C/32) words (5)
+    assert lib.tab_conv2d_workspace_bytes(4, 2, 5, 5, 70) == 2 * 5 * 5 * 2 * 2 * 8
+    assert lib.tab_conv2d_workspace_bytes(5, 2, 5, 5, 70) == 2 * 5 * 5 * 3 * 8
+    assert lib.tab_conv2d_workspace_bytes(6, 2, 5, 5, 70) == 0
+    assert [lib.tab_operand_words(t, 0, 70) for t in range(7)] == [4, 4, 2, 2, 4, 3, 0]
+    assert [lib.tab_operand_words(t, 1, 70) for t in range(7)] == [4, 2, 4, 2, 4, 3, 0]
+    assert lib.tab_operand_words(0, 2, 70) == 0
 
 
 def test_c_abi_rejects_bad_arguments_without_launching():
@@ -55,7 +61,7 @@ def test_c_abi_rejects_bad_arguments_without_launching():
     conv = lambda **kw: lib.tab_conv2d(  # noqa: E731
         kw.get("x", p), p, p, p, kw.get("type", 0), kw.get("p1", 1), 1, kw.get("s1", 1), 1,
         1, kw.get("H", 8), 8, 64, 4, 3, 3, p, kw.get("ws", p), kw.get("ws_bytes", 1 << 20), None)
-    assert conv(type=4) == -1
+    assert conv(type=6) == -1 and conv(type=-1) == -1
     assert conv(s1=0) == -1
     assert conv(p1=-1) == -1
     assert conv(H=1, p1=0) == -2 and b"empty output" in lib.tab_last_error()
@@ -73,6 +79,15 @@ def test_c_abi_rejects_bad_arguments_without_launching():
     assert out(ths=None) == -1
     assert out(qy=None) == -1
     assert out(qy=p + 8, bits=2) == -1 and b"aligned" in lib.tab_last_error()
+    # the CPU-only types: no packed output; type 4 bounds K so that 9 * 64 * K words stays below 2^24
+    assert lib.tab_conv2d_packed_out(p, p, p, 4, 1, 1, 1, 1, 1, 8, 8, 64, 4, 3, 3, p, 1, p, None) == -1
+    assert b"types 0..3" in lib.tab_last_error()
+    assert lib.tab_conv2d_packed(p, p, p, 4, 0, 0, 1, 1, 1, 4, 4, 64 * 29200, 4, 1, 1, p, None) == -2
+    assert b"exact accumulation" in lib.tab_last_error()
+    assert lib.tab_conv2d_packed(p, p, p, 5, 0, 0, 1, 1, 1, 4, 4, 32 * 65536, 4, 1, 1, p, None) == -2
+    assert lib.tab_quantize_format(p, p, 3, 1, 1, 1, 64, p, None) == -1 and b"4 (DRF) or 5 (RTN)" in lib.tab_last_error()
+    assert lib.tab_quantize_format(p, None, 4, 1, 1, 1, 64, p, None) == -1
+    assert lib.tab_quantize_format(p, p, 5, 1, 0, 1, 64, p, None) == -1
     # threshold: workspace
     assert lib.tab_threshold_workspace_bytes(0, 10) == 0
     assert lib.tab_threshold(p, 4, 100, ctypes.c_float(0.7), p, None, 0, None) == -3
@@ -106,6 +121,9 @@ def test_python_mirror_names_and_input_checks():
                        0, 1, 1, 1, 1, 1, 4, 4, 64, 4, 3, 3)
     assert tab_amd.out_shape(112, 112, 3, 3, 1, 1, 1, 1) == (112, 112)
     assert tab_amd.packed_channels(256) == 4
+    with pytest.raises(RuntimeError, match="X must be a CUDA tensor"):
+        tab_amd.QuantizeFormat(x, ths, 4, 1, 4, 4, 64)
+    assert (tab_amd.DRF, tab_amd.RTN) == (4, 5) and tab_amd.operand_words(5, 0, 64) == 2
 
 
 def test_missing_library_fails_loudly(tmp_path):
