@@ -96,24 +96,27 @@ __device__ __forceinline__ i32x8 expand_levels(uint32_t hi, uint32_t lo)
 }
 
 // Type 5 (TAB_CPU.cpp:362-383): a 32-bit slice holds 16 fields (even bit = nonzero, odd bit = sign).
-// The fields at even positions of the slice fill operand dword 0, those at odd positions dword 1,
-// each as the nibble (sign, 0, nonzero, 0) = +-1 or +-0; a slice is 16 of the 32 elements a lane can
-// feed, the other operand dwords stay zero.
-__device__ __forceinline__ i32x8 expand_fields(uint32_t w)
+// The fields at even positions of the slice fill one operand dword, those at odd positions the next,
+// each as the nibble (sign, 0, nonzero, 0) = +-1 or +-0.  A slice is 16 of the 32 elements a lane
+// feeds, so a lane takes both halves of one word per MFMA and the two half-waves take alternate words.
+__device__ __forceinline__ i32x8 expand_fields(uint32_t lo, uint32_t hi)
 {
     i32x8 r = {0, 0, 0, 0, 0, 0, 0, 0};
-    r[0] = (int)(((w << 1) & kBit1) | ((w << 2) & kBit3));
-    r[1] = (int)(((w >> 1) & kBit1) | (w & kBit3));
+    r[0] = (int)(((lo << 1) & kBit1) | ((lo << 2) & kBit3));
+    r[1] = (int)(((lo >> 1) & kBit1) | (lo & kBit3));
+    r[2] = (int)(((hi << 1) & kBit1) | ((hi << 2) & kBit3));
+    r[3] = (int)(((hi >> 1) & kBit1) | (hi & kBit3));
     return r;
 }
 
-// The FP4 operand of one 32-bit slice: SIDE 0 = activation, 1 = weight; p0, p1 = the slice of plane 0
-// and of the last plane (the same word for one-plane operands).
+// The FP4 operand of one MFMA: SIDE 0 = activation, 1 = weight; p0, p1 = the lane's 32-bit slice of
+// plane 0 and of the last plane (the same slice for one-plane operands); type 5: the two halves of
+// the lane's word.
 template <int TYPE, int SIDE>
 __device__ __forceinline__ i32x8 expand_operand(uint32_t p0, uint32_t p1, const ExpandConsts &c)
 {
     if (TYPE == 4) return expand_levels(p0, p1);
-    if (TYPE == 5) return expand_fields(p0);
+    if (TYPE == 5) return expand_fields(p0, p1);
     constexpr int PL = SIDE ? Planes<TYPE>::B : Planes<TYPE>::A;
     return PL == 2 ? expand_ternary<SIDE>(p0, p1, c) : expand_binary<SIDE>(p0, c);
 }
@@ -129,6 +132,9 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
     static_assert(KCH % KS == 0 && (KS == 1 || (TM == 1 && TN == 1)), "k-split waves share one 32x32 tile");
     constexpr int WPW = KCH / KS;  // words of a chunk each wave multiplies
     constexpr int APL = Planes<TYPE>::A, BPL = Planes<TYPE>::B;
+    static_assert(TYPE != 5 || WPW % 2 == 0, "type 5 multiplies two words per MFMA");
+    constexpr int STEPS = TYPE == 5 ? WPW / 2 : WPW;  // MFMAs per tile pair and chunk
+    constexpr int ASL = TYPE == 5 ? 2 : APL, BSL = TYPE == 5 ? 2 : BPL;
     constexpr int BM = 32 * WM * TM, BN = 32 * WN * TN;
     using Stager = typename std::conditional<INTAP, TapStager<TYPE, BM, BN, INTAP ? KCH : 2>, TileStager<TYPE, BM, BN, KCH>>::type;
     constexpr int A_STRIDE = Stager::A_STRIDE, B_STRIDE = Stager::B_STRIDE;
@@ -176,39 +182,43 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
         // nothing for a ternary operand and +64 per word for binary x binary (the BNN bias below
         // counts them).
         const uint32_t *la = lds + (chunk & 1) * (A_DWORDS + B_DWORDS) + a_off, *lb = la - a_off + A_DWORDS + b_off;
-        uint32_t a_w[WPW][APL][TM], b_w[WPW][BPL][TN];
-        auto read_word = [&](int w) {
-            const int q = 2 * (ks + KS * w) + kb;
+        // one step = one MFMA per tile pair; ASL, BSL = the 32-bit slices a lane reads per operand tile and
+        // step: its half of the word of every plane, or (type 5) both halves of its own word
+        uint32_t a_w[STEPS][ASL][TM], b_w[STEPS][BSL][TN];
+        auto read_step = [&](int w) {
 #pragma unroll
-            for (int pl = 0; pl < APL; pl++)
+            for (int sl = 0; sl < ASL; sl++) {
+                const int slice = TYPE == 5 ? 2 * (ks + KS * (2 * w + kb)) + sl : sl * Q + 2 * (ks + KS * w) + kb;
 #pragma unroll
-                for (int mt = 0; mt < TM; mt++) a_w[w][pl][mt] = la[(pl * Q + q) * A_STRIDE + mt * 32];
+                for (int mt = 0; mt < TM; mt++) a_w[w][sl][mt] = la[slice * A_STRIDE + mt * 32];
+            }
 #pragma unroll
-            for (int pl = 0; pl < BPL; pl++)
+            for (int sl = 0; sl < BSL; sl++) {
+                const int slice = TYPE == 5 ? 2 * (ks + KS * (2 * w + kb)) + sl : sl * Q + 2 * (ks + KS * w) + kb;
 #pragma unroll
-                for (int nt = 0; nt < TN; nt++) b_w[w][pl][nt] = lb[(pl * Q + q) * B_STRIDE + nt * 32];
+                for (int nt = 0; nt < TN; nt++) b_w[w][sl][nt] = lb[slice * B_STRIDE + nt * 32];
+            }
         };
         // LDS reads run ahead of the matrix cores: the whole chunk up front when that is few registers
-        // (one-plane operands; measured +3 % on BNN, a loss for the two-plane types), else one word ahead
-        constexpr bool ALL_AHEAD = (APL * TM + BPL * TN) * WPW <= 16;
+        // (one-plane operands; measured +3 % on BNN, a loss for the two-plane types), else one step ahead
+        constexpr bool ALL_AHEAD = (ASL * TM + BSL * TN) * STEPS <= 16;
         if (ALL_AHEAD) {
 #pragma unroll
-            for (int w = 0; w < WPW; w++) read_word(w);
+            for (int w = 0; w < STEPS; w++) read_step(w);
             __builtin_amdgcn_sched_barrier(0);
         } else {
-            read_word(0);
+            read_step(0);
         }
 #pragma unroll
-        for (int w = 0; w < WPW; w++) {
-            if (!ALL_AHEAD && w + 1 < WPW) read_word(w + 1);
+        for (int w = 0; w < STEPS; w++) {
+            if (!ALL_AHEAD && w + 1 < STEPS) read_step(w + 1);
             i32x8 af[TM], bf[TN];
 #pragma unroll
-            for (int mt = 0; mt < TM; mt++)
-                af[mt] = expand_operand<TYPE, 0>(a_w[w][0][mt], a_w[w][APL - 1][mt], consts);
+            for (int mt = 0; mt < TM; mt++) af[mt] = expand_operand<TYPE, 0>(a_w[w][0][mt], a_w[w][ASL - 1][mt], consts);
 #pragma unroll
             for (int nt = 0; nt < TN; nt++) {
-                bf[nt] = expand_operand<TYPE, 1>(b_w[w][0][nt], b_w[w][BPL - 1][nt], consts);
-                if (TYPE == 2) b_nonzero[nt] += __builtin_popcount(b_w[w][BPL - 1][nt]);
+                bf[nt] = expand_operand<TYPE, 1>(b_w[w][0][nt], b_w[w][BSL - 1][nt], consts);
+                if (TYPE == 2) b_nonzero[nt] += __builtin_popcount(b_w[w][BSL - 1][nt]);
             }
 #pragma unroll
             for (int mt = 0; mt < TM; mt++)
@@ -395,14 +405,19 @@ hipError_t launch_mfma_shape(const ConvArgs &a, hipStream_t stream)
     if constexpr (LONG)
         if (a.PC % 8 == 0) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 8, true>(a, stream);
     if (a.PC % 4 == 0) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 4, true>(a, stream);
-    if constexpr (LONG)
+    if constexpr (LONG && TYPE != 5)
         if (a.G % 9 == 0) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 9, false>(a, stream);
     if (a.PC % 2 == 0) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 2, true>(a, stream);
-    switch (mfma_chunk_words(a.G)) {
-    case 1: return launch_mfma_tile<TYPE, WM, WN, TM, TN, 1, false>(a, stream);
-    case 2: return launch_mfma_tile<TYPE, WM, WN, TM, TN, 2, false>(a, stream);
-    case 3: return launch_mfma_tile<TYPE, WM, WN, TM, TN, 3, false>(a, stream);
-    default: return launch_mfma_tile<TYPE, WM, WN, TM, TN, 4, false>(a, stream);
+    if constexpr (TYPE == 5) {  // whole pairs of words per chunk
+        if ((a.G + 1) / 2 % 2 == 0) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 4, false>(a, stream);
+        return launch_mfma_tile<TYPE, WM, WN, TM, TN, 2, false>(a, stream);
+    } else {
+        switch (mfma_chunk_words(a.G)) {
+        case 1: return launch_mfma_tile<TYPE, WM, WN, TM, TN, 1, false>(a, stream);
+        case 2: return launch_mfma_tile<TYPE, WM, WN, TM, TN, 2, false>(a, stream);
+        case 3: return launch_mfma_tile<TYPE, WM, WN, TM, TN, 3, false>(a, stream);
+        default: return launch_mfma_tile<TYPE, WM, WN, TM, TN, 4, false>(a, stream);
+        }
     }
 }
 
@@ -421,9 +436,13 @@ hipError_t launch_mfma_type(const ConvArgs &a, int shape, hipStream_t stream)
     case 6: return launch_mfma_shape<TYPE, 2, 2, 2, 4>(a, stream);
     case 3:
         if (a.PC % 8 == 0) return launch_mfma_tile<TYPE, 1, 1, 1, 1, 8, true, 4>(a, stream);
-        if (a.PC % 4 == 0) return launch_mfma_tile<TYPE, 1, 1, 1, 1, 4, true, 4>(a, stream);
-        if (a.G > 4) return launch_mfma_tile<TYPE, 1, 1, 1, 1, 12, false, 4>(a, stream);
-        return launch_mfma_tile<TYPE, 1, 1, 1, 1, 4, false, 4>(a, stream);
+        if constexpr (TYPE == 5) {  // two words per wave and chunk at least
+            return launch_mfma_tile<TYPE, 1, 1, 1, 1, 8, false, 4>(a, stream);
+        } else {
+            if (a.PC % 4 == 0) return launch_mfma_tile<TYPE, 1, 1, 1, 1, 4, true, 4>(a, stream);
+            if (a.G > 4) return launch_mfma_tile<TYPE, 1, 1, 1, 1, 12, false, 4>(a, stream);
+            return launch_mfma_tile<TYPE, 1, 1, 1, 1, 4, false, 4>(a, stream);
+        }
     default: return hipErrorInvalidValue;
     }
 }

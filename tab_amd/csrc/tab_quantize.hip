@@ -43,9 +43,11 @@ __device__ __forceinline__ int wave_sum(int v)
 }
 
 // Compare one float4 against the threshold; bit e of the result belongs to element e.
-// Ternary: first test v > t (+1), only then v < -t (-1); both are strict and ordered, so
-// ties and NaN give 0 (TAB_GEMM.cu:184-192).  Binary: bit = v < t (TAB_GEMM.cu:231).
-template <int BITS>
+// MODE 2, ternary: first test v > t (+1), only then v < -t (-1); both are strict and ordered, so
+// ties and NaN give 0 (TAB_GEMM.cu:184-192).  MODE 1, binary: bit = v < t (TAB_GEMM.cu:231).
+// MODE 5 (RTN fields) compares like MODE 2.  MODE 4 (2-bit levels): `sign` gets the weight-2 bit and
+// `nz` the weight-1 bit of level = (v >= 0.5t) + (v >= 1.5t) + (v >= 2.5t).
+template <int MODE>
 __device__ __forceinline__ void compare4(const floatx4 v, const float t, uint32_t &sign, uint32_t &nz)
 {
     const float e[4] = {v[0], v[1], v[2], v[3]};
@@ -53,22 +55,57 @@ __device__ __forceinline__ void compare4(const floatx4 v, const float t, uint32_
     nz = 0;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        if (BITS == 2) {
+        if (MODE == 2 || MODE == 5) {
             const bool pos = e[i] > t;
             const bool neg = !pos && (e[i] < -t);
             nz |= (uint32_t)(pos || neg) << i;
             sign |= (uint32_t)neg << i;
+        } else if (MODE == 4) {
+            const int level = (int)(e[i] >= 0.5f * t) + (int)(e[i] >= 1.5f * t) + (int)(e[i] >= 2.5f * t);
+            sign |= (uint32_t)(level >> 1) << i;
+            nz |= (uint32_t)(level & 1) << i;
         } else {
             sign |= (uint32_t)(e[i] < t) << i;
         }
     }
 }
 
+// The packed output of one 64-channel row from the compare bits of lane l of its 16-lane DPP row; all
+// lanes of the row take part, lane 0 gets the complete result: out[0..1] for MODE 1, out[0..3] else.
+// MODE 1/2/4: the lane's nibble goes to bit 4*(l%8) and an OR over 8 lanes yields the low (lanes 0-7)
+// or high (lanes 8-15) 32 bits of a plane word; a rotate by 8 within the row hands lane 0 the other
+// half: (plane 0 low, plane 0 high, plane 1 low, plane 1 high).
+// MODE 5: the row is two words of 32 two-bit fields (TAB_CPU.cpp:364-379); the lane's four fields
+// (8 bits, even bit = nonzero, odd bit = sign) go to byte l%4 of the low (l%8 < 4) or high half of the
+// word lanes 0-7 (channels 0-31) or lanes 8-15 (channels 32-63) build: (word 0 low, high, word 1 low, high).
+template <int MODE>
+__device__ __forceinline__ void pack_row(uint32_t sign, uint32_t nz, int l, uint32_t (&out)[4])
+{
+    if (MODE == 5) {
+        uint32_t fields = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) fields |= (((nz >> i) & 1u) | (((sign >> i) & 1u) << 1)) << (2 * i);
+        const uint32_t placed = fields << (8 * (l & 3));
+        const uint32_t lo = or_reduce8((l & 4) ? 0u : placed), hi = or_reduce8((l & 4) ? placed : 0u);
+        out[0] = lo; out[1] = hi; out[2] = rotate_row8(lo); out[3] = rotate_row8(hi);
+        return;
+    }
+    const int shift = 4 * (l & 7);
+    const uint32_t sign_half = or_reduce8(sign << shift);
+    out[0] = sign_half;
+    out[1] = rotate_row8(sign_half);
+    if (MODE != 1) {
+        const uint32_t nz_half = or_reduce8(nz << shift);
+        out[2] = nz_half;
+        out[3] = rotate_row8(nz_half);
+    }
+}
+
 // Fast path, C % 64 == 0 and X 16-byte aligned.
 // Lane layout: a 16-lane DPP row reads one 64-channel row as 16 float4 (256 B contiguous),
 // a wave reads 4 consecutive rows per load (1 KB contiguous) and keeps kLoadsPerLane loads
-// in flight.  Each lane turns its 4 compares into a nibble placed at bit 4*(lane%8); an OR
-// over 8 lanes yields the low (lanes 0-7) or high (lanes 8-15) 32 bits of the word.
+// in flight; pack_row turns the compare bits of the row's lanes into its packed element.
+// BITS = 1 or 2 (the reference's bit widths), or the format of conv type 4 or 5.
 template <int BITS>
 __global__ __launch_bounds__(kThreads) void quantize_rows64(const floatx4 *__restrict__ x,
                                                             const float *__restrict__ ths,
@@ -100,21 +137,13 @@ __global__ __launch_bounds__(kThreads) void quantize_rows64(const floatx4 *__res
         const long r = row0 + u * 4 + sub;
         float t = t_first;
         if (!one_item) t = ths[(r < rows ? r : rows - 1) / rows_per_item];
-        uint32_t sign, nz;
+        uint32_t sign, nz, out[4];
         compare4<BITS>(v[u], t, sign, nz);
-        const int shift = 4 * (l & 7);
-        // after the reduction lanes 0-7 of the row hold the low half, lanes 8-15 the high half;
-        // a rotate by 8 within the row hands lane 0 the other half, and lane 0 stores the whole
-        // element (8 or 16 bytes) at once
-        const uint32_t sign_half = or_reduce8(sign << shift);
-        const uint32_t sign_other = rotate_row8(sign_half);
-        if (BITS == 2) {
-            const uint32_t nz_half = or_reduce8(nz << shift);
-            const uint32_t nz_other = rotate_row8(nz_half);
-            if (r < rows && l == 0)
-                *reinterpret_cast<uintx4 *>(q + r * 4) = uintx4{sign_half, sign_other, nz_half, nz_other};
+        pack_row<BITS>(sign, nz, l, out);  // lane 0 stores the whole element (8 or 16 bytes) at once
+        if (BITS != 1) {
+            if (r < rows && l == 0) *reinterpret_cast<uintx4 *>(q + r * 4) = uintx4{out[0], out[1], out[2], out[3]};
         } else {
-            if (r < rows && l == 0) *reinterpret_cast<uintx2 *>(q + r * 2) = uintx2{sign_half, sign_other};
+            if (r < rows && l == 0) *reinterpret_cast<uintx2 *>(q + r * 2) = uintx2{out[0], out[1]};
         }
     }
 }
@@ -149,18 +178,13 @@ __global__ __launch_bounds__(64) void quantize_rows64_strided(const floatx4 *__r
     for (int u = 0; u < kLoadsPerLane; u++) {
         const int j = j0 + u * 4 + sub;
         const long r = out_line + j;
-        uint32_t sign, nz;
+        uint32_t sign, nz, out[4];
         compare4<BITS>(v[u], t, sign, nz);
-        const int shift = 4 * (l & 7);
-        const uint32_t sign_half = or_reduce8(sign << shift);
-        const uint32_t sign_other = rotate_row8(sign_half);
-        if (BITS == 2) {
-            const uint32_t nz_half = or_reduce8(nz << shift);
-            const uint32_t nz_other = rotate_row8(nz_half);
-            if (j < line_words && l == 0)
-                *reinterpret_cast<uintx4 *>(q + r * 4) = uintx4{sign_half, sign_other, nz_half, nz_other};
+        pack_row<BITS>(sign, nz, l, out);
+        if (BITS != 1) {
+            if (j < line_words && l == 0) *reinterpret_cast<uintx4 *>(q + r * 4) = uintx4{out[0], out[1], out[2], out[3]};
         } else {
-            if (j < line_words && l == 0) *reinterpret_cast<uintx2 *>(q + r * 2) = uintx2{sign_half, sign_other};
+            if (j < line_words && l == 0) *reinterpret_cast<uintx2 *>(q + r * 2) = uintx2{out[0], out[1]};
         }
     }
 }
@@ -404,6 +428,21 @@ hipError_t launch_quantize_format(const float *x, const float *ths, int format, 
 {
     const int PC = format == 5 ? (C + 31) / 32 : (C + kWordBits - 1) / kWordBits;
     const long pixels = items * pixels_per_item;
+    if (format != 4 && format != 5) return hipErrorInvalidValue;
+    if ((C % kWordBits == 0) && ((uintptr_t)x % 16 == 0)) {
+        // whole 64-channel rows: the streaming kernel; a row is 16 bytes of either format
+        const long rows = pixels * (C / kWordBits);
+        const long blocks = (rows + kRowsPerWave * kWavesPerBlock - 1) / (kRowsPerWave * kWavesPerBlock);
+        const dim3 grid((unsigned)blocks), block(kThreads);
+        const floatx4 *x4 = reinterpret_cast<const floatx4 *>(x);
+        uint32_t *q32 = reinterpret_cast<uint32_t *>(qx);
+        const long rows_per_item = pixels_per_item * (C / kWordBits);
+        if (format == 4)
+            quantize_rows64<4><<<grid, block, 0, stream>>>(x4, ths, q32, rows, rows_per_item);
+        else
+            quantize_rows64<5><<<grid, block, 0, stream>>>(x4, ths, q32, rows, rows_per_item);
+        return hipGetLastError();
+    }
     const long units = pixels * PC;
     long blocks = (units + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks > 256 * 32) blocks = 256 * 32;  // grid-stride beyond 32 blocks per CU
