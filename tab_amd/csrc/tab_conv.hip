@@ -351,29 +351,28 @@ hipError_t launch_conv_mfma(int type, const ConvArgs &args, int shape, hipStream
 }
 
 // Workgroup tile of the matrix-core kernel, from measurements over the ResNet-18, VGG and sweep layers at
-// N = 8 .. 256: the 128-row tiles win as soon as there is about one of them per CU (the 128x128 one
-// with short K they need about four per CU); below roughly 200 workgroups of 64x64 the launch is
-// latency-bound and the k-split 32x32 shape wins.
+// N = 8 .. 256: the 128-row tiles win as soon as there is about one of them per CU (with short K the
+// 128x128 one needs several per CU); below roughly 200 workgroups of 64x64 the launch is latency-bound
+// and the k-split 32x32 shape wins.
 int conv_mfma_shape(int conv_type, const ConvArgs &a)
 {
     // the CPU-only types follow the type with the same planes: 4 like TNN, 5 like BNN
     const int type = conv_type == 4 ? 0 : (conv_type == 5 ? 3 : conv_type);
     auto tiles = [&](int bm, int bn) { return (long)((a.M + bm - 1) / bm) * ((a.KN + bn - 1) / bn); };
-    const long enough = a.G >= 36 ? 300 : 1024;  // short K: the per-tile prologue and epilogue weigh more
+    // short K: the per-tile prologue and epilogue weigh more, so a shape needs more tiles to pay
+    const long enough = a.G >= 72 ? 192 : (a.G >= 36 ? 300 : 1024);
     // eight tiles per wave share each expanded operand between more MFMAs (the dearer operand gets the
-    // 4-tile side): +4-13 % for the types with a two-plane operand (nothing for BNN), but only when the
-    // launch is many rounds of these big tiles, or fits in one
-    if (a.G >= 36 && type != 3) {
-        const long big = tiles(256, 128);
-        if (big >= 2560 || (big >= 300 && big <= 512)) {
-            if (type == 1 && a.KN >= 256) return 6;
-            if (type != 1 && a.KN >= 128) return 5;
-        }
+    // 4-tile side): +2-18 %, but only when the launch is many rounds of these big tiles
+    if (a.G >= 36 && tiles(256, 128) >= 2560) {
+        if (type == 1 && a.KN >= 256) return 6;
+        if (type != 1 && a.KN >= 128) return 5;
     }
-    if (a.KN > 64 && a.G >= 18 && tiles(128, 128) >= enough) return 0;
+    if (a.KN > 64 && tiles(128, 128) >= (a.G >= 18 ? enough : 4096)) return 0;
     // one tile of filters: 256 rows per workgroup halve the expansions per MFMA of the 128x64 shape (two-plane
     // operands gain 20 %, BNN nothing)
     if (a.KN <= 64 && type != 3 && tiles(256, 64) >= 1024) return 4;
+    // a handful of words of K (1x1 layers on few channels): the 64x64 shape's short prologue wins
+    if (a.G <= 4 && tiles(64, 64) >= 192) return 2;
     if (tiles(128, 64) >= enough) return 1;
     if (tiles(64, 64) >= 192 || a.qy != nullptr) return 2;  // the packed epilogue needs tiles 64 filters wide
     return 3;

@@ -121,117 +121,15 @@ __device__ __forceinline__ i32x8 expand_operand(uint32_t p0, uint32_t p1, const 
     return PL == 2 ? expand_ternary<SIDE>(p0, p1, c) : expand_binary<SIDE>(p0, c);
 }
 
-// waves_per_eu: the shapes with four MFMA tiles per wave are capped at 128 registers, i.e. four
-// workgroups per CU (the 128x128 shape otherwise takes 136-152, 64 of them accumulators, and runs
-// three, measured 3-7 % slower); 256-row tiles need the state of more staged rows and get 168
-// (three workgroups), eight tiles per wave 256 (two).
-template <int TYPE, int WM, int WN, int TM, int TN, int KCH, bool INTAP, int KS = 1>
-__global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM * TN > 4 ? 2 : (WM * TM > 4 ? 3 : 4)))) void conv_mfma(const ConvArgs p)
+// Epilogue shared by the matrix-core kernels: accumulator element 4*j + i of lane (kb, r) is
+// C[8*j + 4*kb + i][r] of the wave's 32x32 tile (mt, nt).  b_nonzero: BTN, bits set in the nonzero plane of
+// the k-positions this lane multiplied, per filter tile; partial: KS * 17 * 64 floats of LDS when the KS
+// waves of the workgroup hold partial sums of one tile.
+template <int TYPE, int TM, int TN, int KCH, int KS>
+__device__ __forceinline__ void conv_mfma_epilogue(const ConvArgs &p, f32x16 (&acc)[TM][TN], int (&b_nonzero)[TN], int wave_m0,
+                                                   int wave_n0, int lane, int ks, float *partial)
 {
-    static_assert(WM * WN * KS * 64 == kConvThreads, "four waves");
-    static_assert(KCH % KS == 0 && (KS == 1 || (TM == 1 && TN == 1)), "k-split waves share one 32x32 tile");
-    constexpr int WPW = KCH / KS;  // words of a chunk each wave multiplies
-    constexpr int APL = Planes<TYPE>::A, BPL = Planes<TYPE>::B;
-    static_assert(TYPE != 5 || WPW % 2 == 0, "type 5 multiplies two words per MFMA");
-    constexpr int STEPS = TYPE == 5 ? WPW / 2 : WPW;  // MFMAs per tile pair and chunk
-    constexpr int ASL = TYPE == 5 ? 2 : APL, BSL = TYPE == 5 ? 2 : BPL;
-    constexpr int BM = 32 * WM * TM, BN = 32 * WN * TN;
-    using Stager = typename std::conditional<INTAP, TapStager<TYPE, BM, BN, INTAP ? KCH : 2>, TileStager<TYPE, BM, BN, KCH>>::type;
-    constexpr int A_STRIDE = Stager::A_STRIDE, B_STRIDE = Stager::B_STRIDE;
-    constexpr int Q = Stager::Q, A_DWORDS = Stager::A_DWORDS, B_DWORDS = Stager::B_DWORDS;
-
-    __shared__ __attribute__((aligned(16))) uint32_t lds[2 * (A_DWORDS + B_DWORDS)];
-    __shared__ float partial[KS > 1 ? KS * 17 * 64 : 1];  // k-split: 16 accumulators + the BTN count per lane
-
-    const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63;
-    const int r = lane & 31;   // row of an A tile / column of a B tile
-    const int kb = lane >> 5;  // which 32-bit half of the word this lane feeds
-    const int ks = wave / (WM * WN);  // which words of every chunk this wave takes
-    const int wm = (wave % (WM * WN)) % WM, wn = (wave % (WM * WN)) / WM;
-    const int tile_m = blockIdx.x % p.tiles_m, tile_n = blockIdx.x / p.tiles_m;
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
-
-    Stager st;
-    st.init(p, tid, m0, n0);
-    const ExpandConsts consts;
-
-    f32x16 acc[TM][TN];
-#pragma unroll
-    for (int mt = 0; mt < TM; mt++)
-#pragma unroll
-        for (int nt = 0; nt < TN; nt++)
-#pragma unroll
-            for (int e = 0; e < 16; e++) acc[mt][nt][e] = 0.f;
-    int b_nonzero[TN];  // BTN: bits set in the nonzero plane of this lane's half of its filters
-#pragma unroll
-    for (int nt = 0; nt < TN; nt++) b_nonzero[nt] = 0;
-
-    const int wave_m0 = m0 + wm * (32 * TM), wave_n0 = n0 + wn * (32 * TN);
-
-    st.fetch(p, 0);
-    st.stage(lds);
-    __syncthreads();
-
-    const int a_off = wm * (32 * TM) + r, b_off = wn * (32 * TN) + r;
-    for (int chunk = 0; chunk < p.nchunks; chunk++) {
-        const bool more = chunk + 1 < p.nchunks;
-        if (more) st.fetch(p, chunk + 1);
-
-        // Every chunk is exactly KCH words: the stager zero-fills words past the end of K, which add
-        // nothing for a ternary operand and +64 per word for binary x binary (the BNN bias below
-        // counts them).
-        const uint32_t *la = lds + (chunk & 1) * (A_DWORDS + B_DWORDS) + a_off, *lb = la - a_off + A_DWORDS + b_off;
-        // one step = one MFMA per tile pair; ASL, BSL = the 32-bit slices a lane reads per operand tile and
-        // step: its half of the word of every plane, or (type 5) both halves of its own word
-        uint32_t a_w[STEPS][ASL][TM], b_w[STEPS][BSL][TN];
-        auto read_step = [&](int w) {
-#pragma unroll
-            for (int sl = 0; sl < ASL; sl++) {
-                const int slice = TYPE == 5 ? 2 * (ks + KS * (2 * w + kb)) + sl : sl * Q + 2 * (ks + KS * w) + kb;
-#pragma unroll
-                for (int mt = 0; mt < TM; mt++) a_w[w][sl][mt] = la[slice * A_STRIDE + mt * 32];
-            }
-#pragma unroll
-            for (int sl = 0; sl < BSL; sl++) {
-                const int slice = TYPE == 5 ? 2 * (ks + KS * (2 * w + kb)) + sl : sl * Q + 2 * (ks + KS * w) + kb;
-#pragma unroll
-                for (int nt = 0; nt < TN; nt++) b_w[w][sl][nt] = lb[slice * B_STRIDE + nt * 32];
-            }
-        };
-        // LDS reads run ahead of the matrix cores: the whole chunk up front when that is few registers
-        // (one-plane operands; measured +3 % on BNN, a loss for the two-plane types), else one step ahead
-        constexpr bool ALL_AHEAD = (ASL * TM + BSL * TN) * STEPS <= 16;
-        if (ALL_AHEAD) {
-#pragma unroll
-            for (int w = 0; w < STEPS; w++) read_step(w);
-            __builtin_amdgcn_sched_barrier(0);
-        } else {
-            read_step(0);
-        }
-#pragma unroll
-        for (int w = 0; w < STEPS; w++) {
-            if (!ALL_AHEAD && w + 1 < STEPS) read_step(w + 1);
-            i32x8 af[TM], bf[TN];
-#pragma unroll
-            for (int mt = 0; mt < TM; mt++) af[mt] = expand_operand<TYPE, 0>(a_w[w][0][mt], a_w[w][ASL - 1][mt], consts);
-#pragma unroll
-            for (int nt = 0; nt < TN; nt++) {
-                bf[nt] = expand_operand<TYPE, 1>(b_w[w][0][nt], b_w[w][BSL - 1][nt], consts);
-                if (TYPE == 2) b_nonzero[nt] += __builtin_popcount(b_w[w][BSL - 1][nt]);
-            }
-#pragma unroll
-            for (int mt = 0; mt < TM; mt++)
-#pragma unroll
-                for (int nt = 0; nt < TN; nt++)
-                    acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[mt], bf[nt], acc[mt][nt], 4, 4, 0, 0, 0, 0);
-        }
-
-        if (more) st.stage(lds + ((chunk + 1) & 1) * (A_DWORDS + B_DWORDS));
-        __syncthreads();
-    }
-
-    // ---- epilogue: accumulator element 4*j + i of lane (kb, r) is C[8*j + 4*kb + i][r] -------
+    const int r = lane & 31, kb = lane >> 5;
     // btn of this lane's filters (BTN) and, for packed output, the threshold of row r of each 32-row
     // tile; loaded here rather than before the loop because the registers they would hold through
     // it push the 128x128 shape over its 128-register budget (requesting them early gained nothing)
@@ -371,6 +269,119 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
     }
 }
 
+// waves_per_eu: the shapes with four MFMA tiles per wave are capped at 128 registers, i.e. four
+// workgroups per CU (the 128x128 shape otherwise takes 136-152, 64 of them accumulators, and runs
+// three, measured 3-7 % slower); 256-row tiles need the state of more staged rows and get 168
+// (three workgroups), eight tiles per wave 256 (two).
+template <int TYPE, int WM, int WN, int TM, int TN, int KCH, bool INTAP, int KS = 1>
+__global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM * TN > 4 ? 2 : (WM * TM > 4 ? 3 : 4)))) void conv_mfma(const ConvArgs p)
+{
+    static_assert(WM * WN * KS * 64 == kConvThreads, "four waves");
+    static_assert(KCH % KS == 0 && (KS == 1 || (TM == 1 && TN == 1)), "k-split waves share one 32x32 tile");
+    constexpr int WPW = KCH / KS;  // words of a chunk each wave multiplies
+    constexpr int APL = Planes<TYPE>::A, BPL = Planes<TYPE>::B;
+    static_assert(TYPE != 5 || WPW % 2 == 0, "type 5 multiplies two words per MFMA");
+    constexpr int STEPS = TYPE == 5 ? WPW / 2 : WPW;  // MFMAs per tile pair and chunk
+    constexpr int ASL = TYPE == 5 ? 2 : APL, BSL = TYPE == 5 ? 2 : BPL;
+    constexpr int BM = 32 * WM * TM, BN = 32 * WN * TN;
+    using Stager = typename std::conditional<INTAP, TapStager<TYPE, BM, BN, INTAP ? KCH : 2>, TileStager<TYPE, BM, BN, KCH>>::type;
+    constexpr int A_STRIDE = Stager::A_STRIDE, B_STRIDE = Stager::B_STRIDE;
+    constexpr int Q = Stager::Q, A_DWORDS = Stager::A_DWORDS, B_DWORDS = Stager::B_DWORDS;
+
+    __shared__ __attribute__((aligned(16))) uint32_t lds[2 * (A_DWORDS + B_DWORDS)];
+    __shared__ float partial[KS > 1 ? KS * 17 * 64 : 1];  // k-split: 16 accumulators + the BTN count per lane
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int r = lane & 31;   // row of an A tile / column of a B tile
+    const int kb = lane >> 5;  // which 32-bit half of the word this lane feeds
+    const int ks = wave / (WM * WN);  // which words of every chunk this wave takes
+    const int wm = (wave % (WM * WN)) % WM, wn = (wave % (WM * WN)) / WM;
+    const int tile_m = blockIdx.x % p.tiles_m, tile_n = blockIdx.x / p.tiles_m;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    Stager st;
+    st.init(p, tid, m0, n0);
+    const ExpandConsts consts;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int mt = 0; mt < TM; mt++)
+#pragma unroll
+        for (int nt = 0; nt < TN; nt++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[mt][nt][e] = 0.f;
+    int b_nonzero[TN];  // BTN: bits set in the nonzero plane of this lane's half of its filters
+#pragma unroll
+    for (int nt = 0; nt < TN; nt++) b_nonzero[nt] = 0;
+
+    const int wave_m0 = m0 + wm * (32 * TM), wave_n0 = n0 + wn * (32 * TN);
+
+    st.fetch(p, 0);
+    st.stage(lds);
+    __syncthreads();
+
+    const int a_off = wm * (32 * TM) + r, b_off = wn * (32 * TN) + r;
+    for (int chunk = 0; chunk < p.nchunks; chunk++) {
+        const bool more = chunk + 1 < p.nchunks;
+        if (more) st.fetch(p, chunk + 1);
+
+        // Every chunk is exactly KCH words: the stager zero-fills words past the end of K, which add
+        // nothing for a ternary operand and +64 per word for binary x binary (the BNN bias below
+        // counts them).
+        const uint32_t *la = lds + (chunk & 1) * (A_DWORDS + B_DWORDS) + a_off, *lb = la - a_off + A_DWORDS + b_off;
+        // one step = one MFMA per tile pair; ASL, BSL = the 32-bit slices a lane reads per operand tile and
+        // step: its half of the word of every plane, or (type 5) both halves of its own word
+        uint32_t a_w[STEPS][ASL][TM], b_w[STEPS][BSL][TN];
+        auto read_step = [&](int w) {
+#pragma unroll
+            for (int sl = 0; sl < ASL; sl++) {
+                const int slice = TYPE == 5 ? 2 * (ks + KS * (2 * w + kb)) + sl : sl * Q + 2 * (ks + KS * w) + kb;
+#pragma unroll
+                for (int mt = 0; mt < TM; mt++) a_w[w][sl][mt] = la[slice * A_STRIDE + mt * 32];
+            }
+#pragma unroll
+            for (int sl = 0; sl < BSL; sl++) {
+                const int slice = TYPE == 5 ? 2 * (ks + KS * (2 * w + kb)) + sl : sl * Q + 2 * (ks + KS * w) + kb;
+#pragma unroll
+                for (int nt = 0; nt < TN; nt++) b_w[w][sl][nt] = lb[slice * B_STRIDE + nt * 32];
+            }
+        };
+        // LDS reads run ahead of the matrix cores: the whole chunk up front when that is few registers
+        // (one-plane operands; measured +3 % on BNN, a loss for the two-plane types), else one step ahead
+        constexpr bool ALL_AHEAD = (ASL * TM + BSL * TN) * STEPS <= 16;
+        if (ALL_AHEAD) {
+#pragma unroll
+            for (int w = 0; w < STEPS; w++) read_step(w);
+            __builtin_amdgcn_sched_barrier(0);
+        } else {
+            read_step(0);
+        }
+#pragma unroll
+        for (int w = 0; w < STEPS; w++) {
+            if (!ALL_AHEAD && w + 1 < STEPS) read_step(w + 1);
+            i32x8 af[TM], bf[TN];
+#pragma unroll
+            for (int mt = 0; mt < TM; mt++) af[mt] = expand_operand<TYPE, 0>(a_w[w][0][mt], a_w[w][ASL - 1][mt], consts);
+#pragma unroll
+            for (int nt = 0; nt < TN; nt++) {
+                bf[nt] = expand_operand<TYPE, 1>(b_w[w][0][nt], b_w[w][BSL - 1][nt], consts);
+                if (TYPE == 2) b_nonzero[nt] += __builtin_popcount(b_w[w][BSL - 1][nt]);
+            }
+#pragma unroll
+            for (int mt = 0; mt < TM; mt++)
+#pragma unroll
+                for (int nt = 0; nt < TN; nt++)
+                    acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[mt], bf[nt], acc[mt][nt], 4, 4, 0, 0, 0, 0);
+        }
+
+        if (more) st.stage(lds + ((chunk + 1) & 1) * (A_DWORDS + B_DWORDS));
+        __syncthreads();
+    }
+
+    conv_mfma_epilogue<TYPE, TM, TN, KCH, KS>(p, acc, b_nonzero, wave_m0, wave_n0, lane, ks, partial);
+}
+
 // Chunk length for G words: 1..4, the one with the least padded work (a barrier is priced as half a
 // word), longer chunks on ties.
 inline int mfma_chunk_words(int G)
@@ -396,6 +407,21 @@ hipError_t launch_mfma_tile(ConvArgs a, hipStream_t stream)
     return hipGetLastError();
 }
 
+// Chunks inside one filter tap go from global memory straight into LDS (tab_conv_mfma_direct.h), measured
+// 2-14 % faster than staging them through registers; the k-split shape keeps the piece stager of the kernel
+// above (its chunks are too short to split into pairs of words per wave, and it measured no better).
+template <int TYPE, int WM, int WN, int TM, int TN, int KCH>
+hipError_t launch_mfma_direct(ConvArgs a, hipStream_t stream);
+
+template <int TYPE, int WM, int WN, int TM, int TN, int KCH, int KS = 1>
+hipError_t launch_mfma_intap(const ConvArgs &a, hipStream_t stream)
+{
+    if constexpr (KS == 1)
+        return launch_mfma_direct<TYPE, WM, WN, TM, TN, KCH>(a, stream);
+    else
+        return launch_mfma_tile<TYPE, WM, WN, TM, TN, KCH, true, KS>(a, stream);
+}
+
 // LONG: the launch is small enough to be latency-bound, so prefer few long chunks (fewer serial
 // fetch round trips) over a small LDS footprint.
 template <int TYPE, int WM, int WN, int TM, int TN, bool LONG = false>
@@ -403,11 +429,11 @@ hipError_t launch_mfma_shape(const ConvArgs &a, hipStream_t stream)
 {
     // chunks that stay inside one tap take the piece stager
     if constexpr (LONG)
-        if (a.PC % 8 == 0) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 8, true>(a, stream);
-    if (a.PC % 4 == 0) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 4, true>(a, stream);
+        if (a.PC % 8 == 0) return launch_mfma_intap<TYPE, WM, WN, TM, TN, 8>(a, stream);
+    if (a.PC % 4 == 0) return launch_mfma_intap<TYPE, WM, WN, TM, TN, 4>(a, stream);
     if constexpr (LONG && TYPE != 5)
         if (a.G % 9 == 0) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 9, false>(a, stream);
-    if (a.PC % 2 == 0) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 2, true>(a, stream);
+    if (a.PC % 2 == 0) return launch_mfma_intap<TYPE, WM, WN, TM, TN, 2>(a, stream);
     if constexpr (TYPE == 5) {  // whole pairs of words per chunk
         if ((a.G + 1) / 2 % 2 == 0) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 4, false>(a, stream);
         return launch_mfma_tile<TYPE, WM, WN, TM, TN, 2, false>(a, stream);
@@ -435,11 +461,11 @@ hipError_t launch_mfma_type(const ConvArgs &a, int shape, hipStream_t stream)
     case 5: return launch_mfma_shape<TYPE, 2, 2, 4, 2>(a, stream);
     case 6: return launch_mfma_shape<TYPE, 2, 2, 2, 4>(a, stream);
     case 3:
-        if (a.PC % 8 == 0) return launch_mfma_tile<TYPE, 1, 1, 1, 1, 8, true, 4>(a, stream);
+        if (a.PC % 8 == 0) return launch_mfma_intap<TYPE, 1, 1, 1, 1, 8, 4>(a, stream);
         if constexpr (TYPE == 5) {  // two words per wave and chunk at least
             return launch_mfma_tile<TYPE, 1, 1, 1, 1, 8, false, 4>(a, stream);
         } else {
-            if (a.PC % 4 == 0) return launch_mfma_tile<TYPE, 1, 1, 1, 1, 4, true, 4>(a, stream);
+            if (a.PC % 4 == 0) return launch_mfma_intap<TYPE, 1, 1, 1, 1, 4, 4>(a, stream);
             if (a.G > 4) return launch_mfma_tile<TYPE, 1, 1, 1, 1, 12, false, 4>(a, stream);
             return launch_mfma_tile<TYPE, 1, 1, 1, 1, 4, false, 4>(a, stream);
         }

@@ -1,0 +1,216 @@
+// Matrix-core conv kernel whose operands go from global memory straight into LDS
+// (buffer_load_dwordx4 ... lds): no staging registers, no LDS store instructions, and the next
+// chunk streams in while the matrix cores work on the current one.
+//
+// A chunk is KCH words of one filter tap (PC % KCH == 0, KCH even), moved as 16-byte granules: two
+// words of a one-plane operand, one word (sign low/high, nonzero low/high) of a two-plane operand.
+// An LDS-direct load writes lane i's 16 bytes at base + 16*i, and a lane whose offset is out of
+// range writes zeros (padding taps, rows past M, filters past KN), so granule index = piece * ROWS +
+// row with one wave instruction covering 64 consecutive rows of one piece.
+//
+// Per pair of words p the half-waves take alternate words: lane (kb, r) owns word 2p + kb of row r and
+// multiplies its low half in one MFMA and its high half in the next.  A one-plane operand reads its
+// 8 bytes of the pair's granule (ds_read_b64), a two-plane operand the granule of its word
+// (ds_read_b128); both operands follow the same (word, half) order, so any mix of plane counts agrees
+// on k.
+#pragma once
+#include "tab_conv_mfma.h"
+
+namespace tab {
+namespace {
+
+// 16 bytes per lane from a buffer straight into LDS: lane i's data lands at dst + 16*i (dst is
+// wave-uniform), an out-of-range offset writes zeros.  In a function of its own because the cast to the
+// LDS address space must not appear in the kernel's body, which the host pass also parses.
+__device__ __forceinline__ void load16_to_lds(__amdgpu_buffer_rsrc_t rsrc, uint32_t *dst, uint32_t byte_offset)
+{
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void *)dst, 16, byte_offset, 0, 0, 0);
+}
+
+template <int TYPE, int WM, int WN, int TM, int TN, int KCH>
+__global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM * TN > 4 ? 2 : (WM * TM > 4 ? 3 : 4)))) void conv_mfma_direct(const ConvArgs p)
+{
+    static_assert(WM * WN * 64 == kConvThreads && KCH % 2 == 0, "four waves, whole pairs of words");
+    constexpr int PAIRS = KCH / 2;
+    constexpr int APL = Planes<TYPE>::A, BPL = Planes<TYPE>::B;
+    constexpr int BM = 32 * WM * TM, BN = 32 * WN * TN;
+    constexpr int PA = KCH * APL / 2, PB = KCH * BPL / 2;  // granules per row and chunk
+    constexpr int A_GRANULES = PA * BM, B_GRANULES = PB * BN;
+    constexpr int A_ITEMS = (A_GRANULES + kConvThreads - 1) / kConvThreads, B_ITEMS = (B_GRANULES + kConvThreads - 1) / kConvThreads;
+    constexpr int BUF_DWORDS = 4 * (A_ITEMS + B_ITEMS) * kConvThreads;  // whole wave instructions
+
+    __shared__ __attribute__((aligned(16))) uint32_t lds[2 * BUF_DWORDS];
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int r = lane & 31, kb = lane >> 5;
+    const int wm = wave % WM, wn = wave / WM;
+    const int tile_m = blockIdx.x % p.tiles_m, tile_n = blockIdx.x / p.tiles_m;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    // ---- what this lane fetches: granule idx = tid + i * 256 = piece * ROWS + row -------------------
+    const int pixels = p.OH * p.OW;
+    const int n_first = m0 / pixels;  // uniform
+    const size_t image_words = (size_t)p.H * p.W * p.PC * APL;
+    const size_t a_bytes = (size_t)(p.N - n_first) * image_words * 8;
+    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(p.qx + (size_t)n_first * image_words), 0, a_bytes > 0xffffffffull ? (int)0xffffffffu : (int)a_bytes, kBufferFlags);
+    int ih0[A_ITEMS], iw0[A_ITEMS];
+    uint32_t a_base[A_ITEMS], b_base[B_ITEMS];
+#pragma unroll
+    for (int i = 0; i < A_ITEMS; i++) {
+        const int idx = tid + i * kConvThreads;
+        const int piece = idx / BM, row = idx % BM;
+        const int a_m = m0 + row;
+        const bool live = piece < PA && a_m < p.M;
+        const int mm = live ? a_m : m0;
+        const int n = mm / pixels;
+        const int rem = mm - n * pixels;
+        const int oh = rem / p.OW, ow = rem - oh * p.OW;
+        ih0[i] = live ? oh * p.s1 - p.p1 : -(1 << 30);  // a dead granule fails every bounds check
+        iw0[i] = ow * p.s2 - p.p2;
+        a_base[i] = (uint32_t)((((n - n_first) * p.H + (oh * p.s1 - p.p1)) * p.W + iw0[i]) * p.PC) * (uint32_t)(APL * 8) +
+                    (uint32_t)piece * 16u;
+    }
+    const size_t filter_bytes = (size_t)p.G * BPL * 8;
+    const size_t b_bytes = (size_t)(p.KN - n0) * filter_bytes;
+    const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(p.qw + (size_t)n0 * p.G * BPL), 0, b_bytes > kNoFilter ? (int)kNoFilter : (int)b_bytes, kBufferFlags);
+#pragma unroll
+    for (int i = 0; i < B_ITEMS; i++) {
+        const int idx = tid + i * kConvThreads;
+        const int piece = idx / BN, row = idx % BN;
+        const bool live = piece < PB && (n0 + row) < p.KN;
+        b_base[i] = live ? (uint32_t)row * (uint32_t)filter_bytes + (uint32_t)piece * 16u : kNoFilter;
+    }
+
+    auto fetch = [&](int chunk, uint32_t *buf) {
+        const int g0 = chunk * KCH;  // first word of the chunk; the whole chunk lies in one tap
+        const uint32_t tap = fastdiv((uint32_t)g0, p.div_pc);
+        const int pc = g0 - (int)tap * p.PC;
+        const int kh = (int)fastdiv(tap, p.div_kw);
+        const int kw = (int)tap - kh * p.KW;
+        const uint32_t tap_off = (uint32_t)((kh * p.W + kw) * p.PC + pc) * (uint32_t)(APL * 8);
+#pragma unroll
+        for (int i = 0; i < A_ITEMS; i++) {
+            const bool ok = (unsigned)(ih0[i] + kh) < (unsigned)p.H && (unsigned)(iw0[i] + kw) < (unsigned)p.W;
+            load16_to_lds(a_rsrc, buf + 4 * (i * kConvThreads + wave * 64), ok ? a_base[i] + tap_off : kNoData);
+        }
+        const uint32_t word_off = (uint32_t)g0 * (uint32_t)(BPL * 8);
+#pragma unroll
+        for (int i = 0; i < B_ITEMS; i++)
+            load16_to_lds(b_rsrc, buf + 4 * ((A_ITEMS + i) * kConvThreads + wave * 64),
+                          b_base[i] == kNoFilter ? kNoFilter : b_base[i] + word_off);
+    };
+
+    const ExpandConsts consts;
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int mt = 0; mt < TM; mt++)
+#pragma unroll
+        for (int nt = 0; nt < TN; nt++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[mt][nt][e] = 0.f;
+    int b_nonzero[TN];
+#pragma unroll
+    for (int nt = 0; nt < TN; nt++) b_nonzero[nt] = 0;
+
+    const int wave_m0 = m0 + wm * (32 * TM), wave_n0 = n0 + wn * (32 * TN);
+
+    fetch(0, lds);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+
+    // dword offset of this lane's part of granule (pair 0, its row): one-plane: 8 bytes of the pair's granule;
+    // two-plane: the granule of its own word
+    const int a_row = wm * (32 * TM) + r, b_row = wn * (32 * TN) + r;
+    constexpr int A_PAIR = (APL == 1 ? 1 : 2) * BM * 4, B_PAIR = (BPL == 1 ? 1 : 2) * BN * 4;  // dwords between pairs
+    const int a_off = (APL == 1 ? 4 * a_row + 2 * kb : 4 * (kb * BM + a_row));
+    const int b_off = 4 * A_ITEMS * kConvThreads + (BPL == 1 ? 4 * b_row + 2 * kb : 4 * (kb * BN + b_row));
+
+    for (int chunk = 0; chunk < p.nchunks; chunk++) {
+        const bool more = chunk + 1 < p.nchunks;
+        if (more) fetch(chunk + 1, lds + ((chunk + 1) & 1) * BUF_DWORDS);
+
+        const uint32_t *buf = lds + (chunk & 1) * BUF_DWORDS;
+        uint32_t a_w[2][TM][2 * APL], b_w[2][TN][2 * BPL];  // [low half, high half] of every plane of the lane's word
+        auto read_pair = [&](int pair) {
+#pragma unroll
+            for (int mt = 0; mt < TM; mt++) {
+                const uint32_t *src = buf + a_off + pair * A_PAIR + mt * 32 * 4;
+                if (APL == 1) {
+                    const u32x2 v = *reinterpret_cast<const u32x2 *>(src);
+                    a_w[pair & 1][mt][0] = v[0]; a_w[pair & 1][mt][1] = v[1];
+                } else {
+                    const u32x4 v = *reinterpret_cast<const u32x4 *>(src);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) a_w[pair & 1][mt][e] = v[e];
+                }
+            }
+#pragma unroll
+            for (int nt = 0; nt < TN; nt++) {
+                const uint32_t *src = buf + b_off + pair * B_PAIR + nt * 32 * 4;
+                if (BPL == 1) {
+                    const u32x2 v = *reinterpret_cast<const u32x2 *>(src);
+                    b_w[pair & 1][nt][0] = v[0]; b_w[pair & 1][nt][1] = v[1];
+                } else {
+                    const u32x4 v = *reinterpret_cast<const u32x4 *>(src);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) b_w[pair & 1][nt][e] = v[e];
+                }
+            }
+        };
+        read_pair(0);
+#pragma unroll
+        for (int pair = 0; pair < PAIRS; pair++) {
+            if (pair + 1 < PAIRS) read_pair(pair + 1);
+#pragma unroll
+            for (int h = 0; h < (TYPE == 5 ? 1 : 2); h++) {
+                i32x8 af[TM], bf[TN];
+#pragma unroll
+                for (int mt = 0; mt < TM; mt++) {
+                    const uint32_t *w = a_w[pair & 1][mt];
+                    af[mt] = TYPE == 5 ? expand_operand<TYPE, 0>(w[0], w[1], consts)
+                                       : expand_operand<TYPE, 0>(w[h], w[2 * (APL - 1) + h], consts);
+                }
+#pragma unroll
+                for (int nt = 0; nt < TN; nt++) {
+                    const uint32_t *w = b_w[pair & 1][nt];
+                    bf[nt] = TYPE == 5 ? expand_operand<TYPE, 1>(w[0], w[1], consts)
+                                       : expand_operand<TYPE, 1>(w[h], w[2 * (BPL - 1) + h], consts);
+                    if (TYPE == 2) b_nonzero[nt] += __builtin_popcount(w[2 + h]);
+                }
+#pragma unroll
+                for (int mt = 0; mt < TM; mt++)
+#pragma unroll
+                    for (int nt = 0; nt < TN; nt++)
+                        acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[mt], bf[nt], acc[mt][nt], 4, 4, 0, 0, 0, 0);
+            }
+        }
+
+        // keep the wait at the end of the chunk's MFMAs (the scheduler would hoist it above them, since
+        // only memory operations order it): the next chunk's loads have a whole chunk of work to land in
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0);  // this wave's part of the next chunk has landed
+        __syncthreads();
+    }
+
+    conv_mfma_epilogue<TYPE, TM, TN, KCH, 1>(p, acc, b_nonzero, wave_m0, wave_n0, lane, 0, nullptr);
+}
+
+template <int TYPE, int WM, int WN, int TM, int TN, int KCH>
+hipError_t launch_mfma_direct(ConvArgs a, hipStream_t stream)
+{
+    constexpr int BM = 32 * WM * TM, BN = 32 * WN * TN;
+    if (a.PC % KCH != 0) return hipErrorInvalidValue;
+    a.kcw = KCH;
+    a.nchunks = a.G / KCH;
+    a.tiles_m = (a.M + BM - 1) / BM;
+    const long blocks = (long)a.tiles_m * ((a.KN + BN - 1) / BN);
+    if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
+    conv_mfma_direct<TYPE, WM, WN, TM, TN, KCH><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
+    return hipGetLastError();
+}
+
+}  // namespace
+}  // namespace tab

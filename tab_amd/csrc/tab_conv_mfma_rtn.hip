@@ -1,6 +1,6 @@
 // RTN (type 5) instantiations of the matrix-core conv kernel (one translation unit per type so they
 // compile in parallel).
-#include "tab_conv_mfma.h"
+#include "tab_conv_mfma_direct.h"
 
 namespace tab {
 hipError_t launch_conv_mfma_rtn(const ConvArgs &args, int shape, hipStream_t stream)
