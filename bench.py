@@ -452,7 +452,7 @@ def main():
             del L
         result["sweep_N256_28x28x512_3x3"] = sweep
 
-        # ---- more points of the large-batch sweep (BASELINE configs[4]): conv kernel TOP/s ----
+        # ---- more points of the large-batch sweep (the N = 64..256 benchmark configuration): conv kernel TOP/s ----
         # (C=KN, kernel, stride, pad1, pad2) at 28x28; asymmetric padding as the config asks
         points = [(256, 3, 1, 1, 0), (512, 3, 2, 1, 0), (512, 1, 1, 0, 0), (256, 1, 2, 1, 0)]
         more = {}
@@ -467,7 +467,7 @@ def main():
                 more[layer_name(n_batch, lay)] = row
         result["sweep_more_conv_kernel_tops"] = more
 
-        # ---- TNN VGG-16-style stack at N=32 (BASELINE configs[3]) ---------------------------
+        # ---- TNN VGG-16-style stack at N=32 (the VGG benchmark configuration) ---------------------------
         vgg, vgg_ops, vgg_ms, vgg_call_ms = [], 0, 0.0, 0.0
         for i, (hw, c) in enumerate([(224, 64), (112, 128), (56, 256), (28, 512), (14, 512)]):
             lay = (hw, hw, c, c, 3, 3, 1, 1, 1, 1)

@@ -33,7 +33,7 @@ def _conv_case(type, N, H, W, C, KN, KH, KW, p1, p2, s1, s2, seed=0, relu=False)
 
 @pytest.mark.parametrize("type", [0, 1, 2, 3])
 def test_config1_shape(type):
-    # BASELINE config 1: N=1, 32x32x64 -> 64, 3x3, pad 1, stride 1
+    # the single-image benchmark shape: N=1, 32x32x64 -> 64, 3x3, pad 1, stride 1
     _conv_case(type, 1, 32, 32, 64, 64, 3, 3, 1, 1, 1, 1)
 
 
@@ -60,7 +60,7 @@ def test_edge_shapes(type, case):
 
 
 RESNET18_N16 = [
-    # BASELINE configs 2/3: N=16, 3x3 pad 1 stride 1, plus the stride-2 downsample variants
+    # the ResNet-18 benchmark set: N=16, 3x3 pad 1 stride 1, plus the stride-2 downsample variants
     (16, 56, 56, 64, 64, 3, 3, 1, 1, 1, 1), (16, 28, 28, 128, 128, 3, 3, 1, 1, 1, 1),
     (16, 14, 14, 256, 256, 3, 3, 1, 1, 1, 1), (16, 7, 7, 512, 512, 3, 3, 1, 1, 1, 1),
     (16, 56, 56, 64, 128, 3, 3, 1, 1, 2, 2), (16, 28, 28, 128, 256, 3, 3, 1, 1, 2, 2),

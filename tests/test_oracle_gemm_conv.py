@@ -119,7 +119,7 @@ def test_out_extent_formula(case):
 
 CONV_CASES = [
     # N, H, W, C, KN, KH, KW, p1, p2, s1, s2
-    (1, 32, 32, 64, 64, 3, 3, 1, 1, 1, 1),   # BASELINE config 1 shape
+    (1, 32, 32, 64, 64, 3, 3, 1, 1, 1, 1),   # the single-image benchmark shape
     (2, 7, 7, 64, 8, 3, 3, 1, 1, 2, 2),      # OH differs from PyTorch's formula
     (2, 9, 6, 70, 5, 3, 3, 1, 0, 1, 2),      # C % 64 != 0, asymmetric pad and stride
     (2, 8, 8, 128, 16, 1, 1, 0, 0, 2, 2),    # 1x1 stride 2
