@@ -19,9 +19,11 @@
 // the same bit of the same slice.  All partial sums are integers below 2^24 in magnitude
 // (64*G is bounded by the launcher), hence exact in the fp32 accumulators.
 //
-// Tiling: 256 threads = WM x WN waves, each wave TM x TN MFMA tiles of 32x32; operands are
-// staged in LDS exactly as for the popcount kernel (tab_conv_stage.h).  Per 64-bit word a lane
-// reads the 32-bit half lane/32 selects of its row (A) or column (B), lane%32.
+// Tiling: 256 threads = WM x WN waves, each wave TM x TN MFMA tiles of 32x32.  In the kernel of this file
+// operands are staged in LDS through registers exactly as for the popcount kernel (tab_conv_stage.h), and
+// per 64-bit word a lane reads the 32-bit half lane/32 selects of its row (A) or column (B), lane%32; it
+// serves chunks of K that cross filter taps and the k-split shape.  Chunks inside one tap take the kernel
+// of tab_conv_mfma_direct.h, which shares the expansions and the epilogue defined here.
 #pragma once
 #include "tab_conv_stage.h"
 #include <type_traits>
@@ -427,7 +429,7 @@ hipError_t launch_mfma_intap(const ConvArgs &a, hipStream_t stream)
 template <int TYPE, int WM, int WN, int TM, int TN, bool LONG = false>
 hipError_t launch_mfma_shape(const ConvArgs &a, hipStream_t stream)
 {
-    // chunks that stay inside one tap take the piece stager
+    // chunks that stay inside one tap load LDS directly
     if constexpr (LONG)
         if (a.PC % 8 == 0) return launch_mfma_intap<TYPE, WM, WN, TM, TN, 8>(a, stream);
     if (a.PC % 4 == 0) return launch_mfma_intap<TYPE, WM, WN, TM, TN, 4>(a, stream);
