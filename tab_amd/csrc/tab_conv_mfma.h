@@ -409,8 +409,8 @@ hipError_t launch_mfma_tile(ConvArgs a, hipStream_t stream)
     return hipGetLastError();
 }
 
-// Chunks inside one filter tap go from global memory straight into LDS (tab_conv_mfma_direct.h), measured
-// 2-14 % faster than staging them through registers; the k-split shape keeps the piece stager of the kernel
+// Chunks of whole word pairs that stay inside a filter tap (PC even) go from global memory straight into LDS
+// (tab_conv_mfma_direct.h), measured 2-14 % faster than staging them through registers; the k-split shape keeps the piece stager of the kernel
 // above (its chunks are too short to split into pairs of words per wave, and it measured no better).
 template <int TYPE, int WM, int WN, int TM, int TN, int KCH>
 hipError_t launch_mfma_direct(ConvArgs a, hipStream_t stream);
@@ -433,6 +433,10 @@ hipError_t launch_mfma_shape(const ConvArgs &a, hipStream_t stream)
     if constexpr (LONG)
         if (a.PC % 8 == 0) return launch_mfma_intap<TYPE, WM, WN, TM, TN, 8>(a, stream);
     if (a.PC % 4 == 0) return launch_mfma_intap<TYPE, WM, WN, TM, TN, 4>(a, stream);
+    // PC = 2, 6, 10 ...: chunks of six words across taps rather than one pair of words per barrier (+5-13 %),
+    // unless two two-plane operands would push the big tiles' LDS past four workgroups per CU
+    if constexpr (LONG || Planes<TYPE>::A + Planes<TYPE>::B <= 3)
+        if (a.PC % 2 == 0 && a.G % 6 == 0) return launch_mfma_intap<TYPE, WM, WN, TM, TN, 6>(a, stream);
     if constexpr (LONG && TYPE != 5)
         if (a.G % 9 == 0) return launch_mfma_tile<TYPE, WM, WN, TM, TN, 9, false>(a, stream);
     if (a.PC % 2 == 0) return launch_mfma_intap<TYPE, WM, WN, TM, TN, 2>(a, stream);

@@ -2,8 +2,10 @@
 // (buffer_load_dwordx4 ... lds): no staging registers, no LDS store instructions, and the next
 // chunk streams in while the matrix cores work on the current one.
 //
-// A chunk is KCH words of one filter tap (PC % KCH == 0, KCH even), moved as 16-byte granules: two
-// words of a one-plane operand, one word (sign low/high, nonzero low/high) of a two-plane operand.
+// A chunk is KCH consecutive words of K (KCH even, G % KCH == 0), moved as 16-byte granules: two words of
+// a one-plane operand, one word (sign low/high, nonzero low/high) of a two-plane operand.  The two words
+// of a one-plane activation granule must lie in one filter tap, so PC is even; a chunk may span taps
+// (each wave instruction decodes the tap of its granules, one scalar computation).
 // An LDS-direct load writes lane i's 16 bytes at base + 16*i, and a lane whose offset is out of
 // range writes zeros (padding taps, rows past M, filters past KN), so granule index = piece * ROWS +
 // row with one wave instruction covering 64 consecutive rows of one piece.
@@ -69,8 +71,7 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
         const int oh = rem / p.OW, ow = rem - oh * p.OW;
         ih0[i] = live ? oh * p.s1 - p.p1 : -(1 << 30);  // a dead granule fails every bounds check
         iw0[i] = ow * p.s2 - p.p2;
-        a_base[i] = (uint32_t)((((n - n_first) * p.H + (oh * p.s1 - p.p1)) * p.W + iw0[i]) * p.PC) * (uint32_t)(APL * 8) +
-                    (uint32_t)piece * 16u;
+        a_base[i] = (uint32_t)((((n - n_first) * p.H + (oh * p.s1 - p.p1)) * p.W + iw0[i]) * p.PC) * (uint32_t)(APL * 8);
     }
     const size_t filter_bytes = (size_t)p.G * BPL * 8;
     const size_t b_bytes = (size_t)(p.KN - n0) * filter_bytes;
@@ -84,15 +85,18 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
         b_base[i] = live ? (uint32_t)row * (uint32_t)filter_bytes + (uint32_t)piece * 16u : kNoFilter;
     }
 
+    static_assert(BM % 64 == 0 && BN % 64 == 0, "one wave instruction moves 64 rows of one piece");
     auto fetch = [&](int chunk, uint32_t *buf) {
-        const int g0 = chunk * KCH;  // first word of the chunk; the whole chunk lies in one tap
-        const uint32_t tap = fastdiv((uint32_t)g0, p.div_pc);
-        const int pc = g0 - (int)tap * p.PC;
-        const int kh = (int)fastdiv(tap, p.div_kw);
-        const int kw = (int)tap - kh * p.KW;
-        const uint32_t tap_off = (uint32_t)((kh * p.W + kw) * p.PC + pc) * (uint32_t)(APL * 8);
+        const int g0 = chunk * KCH;  // first word of the chunk
 #pragma unroll
         for (int i = 0; i < A_ITEMS; i++) {
+            // the granule's first word and its tap: the same for the 64 rows this wave instruction moves
+            const int g = g0 + (i * kConvThreads + wave * 64) / BM * (APL == 1 ? 2 : 1);
+            const uint32_t tap = fastdiv((uint32_t)g, p.div_pc);
+            const int pc = g - (int)tap * p.PC;
+            const int kh = (int)fastdiv(tap, p.div_kw);
+            const int kw = (int)tap - kh * p.KW;
+            const uint32_t tap_off = (uint32_t)((kh * p.W + kw) * p.PC + pc) * (uint32_t)(APL * 8);
             const bool ok = (unsigned)(ih0[i] + kh) < (unsigned)p.H && (unsigned)(iw0[i] + kw) < (unsigned)p.W;
             load16_to_lds(a_rsrc, buf + 4 * (i * kConvThreads + wave * 64), ok ? a_base[i] + tap_off : kNoData);
         }
@@ -202,7 +206,7 @@ template <int TYPE, int WM, int WN, int TM, int TN, int KCH>
 hipError_t launch_mfma_direct(ConvArgs a, hipStream_t stream)
 {
     constexpr int BM = 32 * WM * TM, BN = 32 * WN * TN;
-    if (a.PC % KCH != 0) return hipErrorInvalidValue;
+    if (a.G % KCH != 0 || (Planes<TYPE>::A == 1 && a.PC % 2 != 0)) return hipErrorInvalidValue;
     a.kcw = KCH;
     a.nchunks = a.G / KCH;
     a.tiles_m = (a.M + BM - 1) / BM;
