@@ -429,9 +429,11 @@ hipError_t launch_mfma_intap(const ConvArgs &a, hipStream_t stream)
 template <int TYPE, int WM, int WN, int TM, int TN, bool LONG = false>
 hipError_t launch_mfma_shape(const ConvArgs &a, hipStream_t stream)
 {
-    // chunks that stay inside one tap load LDS directly
-    if constexpr (LONG)
+    // whole word pairs inside one tap (PC even) load LDS directly
+    if constexpr (LONG) {
+        if (a.PC % 4 == 0 && a.G % 12 == 0) return launch_mfma_intap<TYPE, WM, WN, TM, TN, 12>(a, stream);
         if (a.PC % 8 == 0) return launch_mfma_intap<TYPE, WM, WN, TM, TN, 8>(a, stream);
+    }
     if (a.PC % 4 == 0) return launch_mfma_intap<TYPE, WM, WN, TM, TN, 4>(a, stream);
     // PC = 2, 6, 10 ...: chunks of six words across taps rather than one pair of words per barrier (+5-13 %),
     // unless two two-plane operands would push the big tiles' LDS past four workgroups per CU
