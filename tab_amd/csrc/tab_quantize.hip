@@ -15,6 +15,7 @@ constexpr int kThreads = 256;
 constexpr int kWavesPerBlock = kThreads / 64;
 constexpr int kLoadsPerLane = 8;                // float4 loads in flight per lane
 constexpr int kRowsPerWave = 4 * kLoadsPerLane; // each wave-wide float4 load covers 4 rows
+constexpr long kSmallLaunchBlocks = 512;        // at or below this many 128-row workgroups a launch is latency-bound
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef uint32_t uintx4 __attribute__((ext_vector_type(4)));
@@ -105,8 +106,9 @@ __device__ __forceinline__ void pack_row(uint32_t sign, uint32_t nz, int l, uint
 // Lane layout: a 16-lane DPP row reads one 64-channel row as 16 float4 (256 B contiguous),
 // a wave reads 4 consecutive rows per load (1 KB contiguous) and keeps kLoadsPerLane loads
 // in flight; pack_row turns the compare bits of the row's lanes into its packed element.
-// BITS = 1 or 2 (the reference's bit widths), or the format of conv type 4 or 5.
-template <int BITS>
+// BITS = 1 or 2 (the reference's bit widths), or the format of conv type 4 or 5; LOADS = 8 (128 rows per
+// workgroup) for streaming, 2 for launches too small to fill the chip.
+template <int BITS, int LOADS = kLoadsPerLane>
 __global__ __launch_bounds__(kThreads) void quantize_rows64(const floatx4 *__restrict__ x,
                                                             const float *__restrict__ ths,
                                                             uint32_t *__restrict__ q, long rows,
@@ -116,14 +118,14 @@ __global__ __launch_bounds__(kThreads) void quantize_rows64(const floatx4 *__res
     const int wave = threadIdx.x >> 6;
     const int sub = lane >> 4;  // which of the 4 rows of a load
     const int l = lane & 15;    // float4 within the row
-    const long row0 = ((long)blockIdx.x * kWavesPerBlock + wave) * kRowsPerWave;
+    const long row0 = ((long)blockIdx.x * kWavesPerBlock + wave) * (4 * LOADS);
     if (row0 >= rows) return;
-    long row_last = row0 + kRowsPerWave - 1;
+    long row_last = row0 + (4 * LOADS) - 1;
     if (row_last > rows - 1) row_last = rows - 1;
 
-    floatx4 v[kLoadsPerLane];
+    floatx4 v[LOADS];
 #pragma unroll
-    for (int u = 0; u < kLoadsPerLane; u++) {
+    for (int u = 0; u < LOADS; u++) {
         const long r = row0 + u * 4 + sub;
         v[u] = (r < rows) ? __builtin_nontemporal_load(&x[r * 16 + l]) : floatx4{0.f, 0.f, 0.f, 0.f};
     }
@@ -133,7 +135,7 @@ __global__ __launch_bounds__(kThreads) void quantize_rows64(const floatx4 *__res
     const float t_first = ths[item_first];
 
 #pragma unroll
-    for (int u = 0; u < kLoadsPerLane; u++) {
+    for (int u = 0; u < LOADS; u++) {
         const long r = row0 + u * 4 + sub;
         float t = t_first;
         if (!one_item) t = ths[(r < rows ? r : rows - 1) / rows_per_item];
@@ -149,10 +151,10 @@ __global__ __launch_bounds__(kThreads) void quantize_rows64(const floatx4 *__res
 }
 
 // The same row quantizer for a 1x1 convolution with stride and no padding, which reads only the
-// pixels (oh*s1, ow*s2): one wave per 32 consecutive words of one output line (n, oh); the packed
+// pixels (oh*s1, ow*s2): one wave per 4*LOADS consecutive words of one output line (n, oh); the packed
 // result is the compact [N][OH][OW][PC] activation, i.e. what the conv reads with stride 1.
-// grid = (ceil(OW*PC / 32), N*OH), one wave per workgroup; OW*PC < 65536 (fastdiv range).
-template <int BITS>
+// grid = (ceil(OW*PC / (4*LOADS)), N*OH), one wave per workgroup; OW*PC < 65536 (fastdiv range).
+template <int BITS, int LOADS = kLoadsPerLane>
 __global__ __launch_bounds__(64) void quantize_rows64_strided(const floatx4 *__restrict__ x, const float *__restrict__ ths,
                                                               uint32_t *__restrict__ q, int H, int W, int PC, int OH,
                                                               int OW, int s1, int s2, FastDiv div_pc)
@@ -163,19 +165,19 @@ __global__ __launch_bounds__(64) void quantize_rows64_strided(const floatx4 *__r
     const int line_words = OW * PC;
     const long in_line = ((long)n * H + (long)oh * s1) * W;   // first input pixel of the line
     const long out_line = (long)blockIdx.y * line_words;
-    const int j0 = blockIdx.x * kRowsPerWave;
+    const int j0 = blockIdx.x * (4 * LOADS);
     const float t = ths[n];
 
-    floatx4 v[kLoadsPerLane];
+    floatx4 v[LOADS];
 #pragma unroll
-    for (int u = 0; u < kLoadsPerLane; u++) {
+    for (int u = 0; u < LOADS; u++) {
         const int j = j0 + u * 4 + sub;
         const int ow = (int)fastdiv((uint32_t)j, div_pc), pc = j - ow * PC;
         const long r = (in_line + (long)ow * s2) * PC + pc;
         v[u] = (j < line_words) ? __builtin_nontemporal_load(&x[r * 16 + l]) : floatx4{0.f, 0.f, 0.f, 0.f};
     }
 #pragma unroll
-    for (int u = 0; u < kLoadsPerLane; u++) {
+    for (int u = 0; u < LOADS; u++) {
         const int j = j0 + u * 4 + sub;
         const long r = out_line + j;
         uint32_t sign, nz, out[4];
@@ -399,13 +401,24 @@ hipError_t launch_quantize(const float *x, const float *ths, int bitwidth, long 
     if (fast) {
         const long rows = pixels * PC;
         const long blocks = (rows + kRowsPerWave * kWavesPerBlock - 1) / (kRowsPerWave * kWavesPerBlock);
-        const dim3 grid((unsigned)blocks), block(kThreads);
+        const dim3 block(kThreads);
         const floatx4 *x4 = reinterpret_cast<const floatx4 *>(x);
         uint32_t *q32 = reinterpret_cast<uint32_t *>(qx);
-        if (bitwidth == 2)
-            quantize_rows64<2><<<grid, block, 0, stream>>>(x4, ths, q32, rows, words_per_item);
-        else
-            quantize_rows64<1><<<grid, block, 0, stream>>>(x4, ths, q32, rows, words_per_item);
+        if (blocks <= kSmallLaunchBlocks) {
+            // a tensor too small to fill the chip with 128-row workgroups: 32 rows per workgroup, two loads per lane
+            // (3.1 MB of fp32: 5.5 -> 4.2 us)
+            const dim3 grid((unsigned)((rows + 8 * kWavesPerBlock - 1) / (8 * kWavesPerBlock)));
+            if (bitwidth == 2)
+                quantize_rows64<2, 2><<<grid, block, 0, stream>>>(x4, ths, q32, rows, words_per_item);
+            else
+                quantize_rows64<1, 2><<<grid, block, 0, stream>>>(x4, ths, q32, rows, words_per_item);
+        } else {
+            const dim3 grid((unsigned)blocks);
+            if (bitwidth == 2)
+                quantize_rows64<2><<<grid, block, 0, stream>>>(x4, ths, q32, rows, words_per_item);
+            else
+                quantize_rows64<1><<<grid, block, 0, stream>>>(x4, ths, q32, rows, words_per_item);
+        }
     } else {
         const long units = pixels * PC;
         long blocks = (units + kWavesPerBlock - 1) / kWavesPerBlock;
@@ -466,9 +479,19 @@ hipError_t launch_quantize_strided(const float *x, const float *ths, int bitwidt
                                    int OW, int s1, int s2, uint64_t *qx, hipStream_t stream)
 {
     const int PC = C / kWordBits;
-    const dim3 grid((unsigned)((OW * PC + kRowsPerWave - 1) / kRowsPerWave), (unsigned)(N * OH)), block(64);
+    const dim3 block(64);
     const floatx4 *x4 = reinterpret_cast<const floatx4 *>(x);
     uint32_t *q32 = reinterpret_cast<uint32_t *>(qx);
+    const long waves = (long)((OW * PC + kRowsPerWave - 1) / kRowsPerWave) * N * OH;
+    if (waves <= kSmallLaunchBlocks * kWavesPerBlock) {  // latency-bound: four times the waves, two loads per lane each
+        const dim3 grid((unsigned)((OW * PC + 7) / 8), (unsigned)(N * OH));
+        if (bitwidth == 2)
+            quantize_rows64_strided<2, 2><<<grid, block, 0, stream>>>(x4, ths, q32, H, W, PC, OH, OW, s1, s2, make_fastdiv(PC));
+        else
+            quantize_rows64_strided<1, 2><<<grid, block, 0, stream>>>(x4, ths, q32, H, W, PC, OH, OW, s1, s2, make_fastdiv(PC));
+        return hipGetLastError();
+    }
+    const dim3 grid((unsigned)((OW * PC + kRowsPerWave - 1) / kRowsPerWave), (unsigned)(N * OH));
     if (bitwidth == 2)
         quantize_rows64_strided<2><<<grid, block, 0, stream>>>(x4, ths, q32, H, W, PC, OH, OW, s1, s2, make_fastdiv(PC));
     else
