@@ -469,6 +469,11 @@ hipError_t launch_mfma_type(const ConvArgs &a, int shape, hipStream_t stream)
     case 5: return launch_mfma_shape<TYPE, 2, 2, 4, 2>(a, stream);
     case 6: return launch_mfma_shape<TYPE, 2, 2, 2, 4>(a, stream);
     case 3:
+        // these launches are latency-bound: few long chunks (three or six words per wave) beat many short ones
+        if constexpr (TYPE != 5) {
+            if (a.G % 24 == 0) return launch_mfma_tile<TYPE, 1, 1, 1, 1, 24, false, 4>(a, stream);
+            if (a.G % 12 == 0) return launch_mfma_tile<TYPE, 1, 1, 1, 1, 12, false, 4>(a, stream);
+        }
         if (a.PC % 8 == 0) return launch_mfma_intap<TYPE, 1, 1, 1, 1, 8, 4>(a, stream);
         if constexpr (TYPE == 5) {  // two words per wave and chunk at least
             return launch_mfma_tile<TYPE, 1, 1, 1, 1, 8, false, 4>(a, stream);
