@@ -50,6 +50,10 @@ EDGE_CASES = [
     (5, 4, 4, 1024, 12, 3, 3, 1, 1, 1, 1),    # long K (144 words)
     (3, 9, 11, 192, 20, 1, 1, 0, 0, 2, 3),    # 1x1, no padding, strides (2, 3): only the pixels read are quantized
     (2, 7, 8, 64, 70, 1, 1, 0, 0, 1, 2),      # 1x1, stride on W only
+    (2, 9, 9, 384, 72, 3, 3, 1, 1, 1, 1),     # PC = 6: chunks of six words across taps
+    (1, 12, 12, 640, 40, 3, 3, 1, 1, 2, 2),   # PC = 10
+    (2, 8, 8, 384, 70, 1, 1, 0, 0, 1, 1),     # PC = 6, K = one tap
+    (3, 6, 6, 768, 33, 3, 3, 1, 1, 1, 1),     # PC = 12, small launch: twelve-word chunks
 ]
 
 
@@ -98,6 +102,7 @@ VARIANT_CASES = [
     (3, 10, 10, 128, 40, 3, 3, 1, 1, 1, 1),    # PC = 2: chunks of two words inside a tap
     (2, 9, 9, 512, 72, 3, 3, 1, 1, 2, 2),      # PC = 8: chunks of four words inside a tap
     (1, 3, 3, 8192, 12, 3, 3, 1, 1, 1, 1),     # K = 73728 bits
+    (2, 10, 10, 384, 136, 3, 3, 1, 1, 1, 1),   # PC = 6: six-word chunks across taps in every tile shape
 ]
 
 
