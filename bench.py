@@ -341,7 +341,7 @@ def main():
     ridge = MFMA_FP4_PEAK_TOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
     achieved_gbs = conv_bytes / conv_ms / 1e6
     hbm_bound = intensity < ridge
-    roofline = {"kernel": "conv_mfma<BNN> (v_mfma_f32_32x32x64_f8f6f4, FP4 operands)",
+    roofline = {"kernel": "conv_mfma_direct<BNN> / conv_mfma<BNN> (v_mfma_f32_32x32x64_f8f6f4, FP4 operands)",
                 "bound": "hbm" if hbm_bound else "mfma",
                 "achieved": round(achieved_gbs if hbm_bound else achieved, 2),
                 "peak": HBM_PEAK_GBS if hbm_bound else MFMA_FP4_PEAK_TOPS,
