@@ -76,6 +76,16 @@ int tab_quantize(const float *dev_X, const float *dev_ths, int bitwidth, int N, 
                  int C, int64_t *dev_QX, int32_t *dev_BTN, void *stream);
 
 /*
+ * tab_quantize on an activation stored NCHW, the layout the reference's CPU quantizers read
+ * (Parallel_Ternarize_NCHWB_to_NHWCB / Parallel_Binarize_NCHW_to_NHWC, TAB_CPU.cpp:20-206; its CPU binding
+ * takes N, C, H, W, TAB_CPU.cpp:621): dev_X fp32 [N][C][H][W]; dev_QX and dev_BTN exactly what tab_quantize
+ * gives for the same values stored NHWC, so the conv entry points take it unchanged and a caller holding
+ * NCHW tensors needs no transposed copy.  No spatial padding is applied here (the conv kernel pads).
+ */
+int tab_quantize_nchw(const float *dev_X, const float *dev_ths, int bitwidth, int N, int C, int H, int W,
+                      int64_t *dev_QX, int32_t *dev_BTN, void *stream);
+
+/*
  * Packers for conv types 4 and 5, activations and weights alike (weights as (N,H,W,C) = (KN,KH,KW,C)).
  * The reference defines the word layouts through DRFGEMM_baseline / RTNGEMM_baseline
  * (TAB_CPU.cpp:332-383) but ships no quantizer for them (TAB_Conv calls Parallel_Binarize_NCHW and

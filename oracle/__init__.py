@@ -141,6 +141,13 @@ def quantize_format(x, ths, type, N, H, W, C):
     return qx
 
 
+def quantize_nchw(x, ths, bitwidth, N, C, H, W):
+    """Quantize of an NCHW tensor, the layout the reference's CPU quantizers read (TAB_CPU.cpp:20-206): the
+    same (N,H,W,PC,bits) words as quantize() on the values stored NHWC."""
+    x = np.ascontiguousarray(_f32(x).reshape(N, C, H, W).transpose(0, 2, 3, 1))
+    return quantize(x, ths, bitwidth, N, H, W, C)
+
+
 def pad(a, N, H, W, D, p1, p2):
     a = _i64(a)
     y = np.empty((N, H + 2 * p1, W + 2 * p2, D), dtype=np.int64)

@@ -85,6 +85,34 @@ def Quantize(X, thresholds, bitwidth, N, H, W, C):
     return [QX, BTN]
 
 
+def QuantizeNCHW(X, thresholds, bitwidth, N, C, H, W):
+    """Quantize on an NCHW fp32 tensor (the layout the reference's CPU quantizers read, TAB_CPU.cpp:20-206, and
+    the argument order of its CPU binding, TAB_CPU.cpp:621): returns [QX, BTN] exactly as
+    Quantize(X.permute(0, 2, 3, 1), thresholds, bitwidth, N, H, W, C) would, without the transposed copy."""
+    _check_input(X, "X")
+    _check_input(thresholds, "thresholds")
+    _check_dtype(X, torch.float32, "X")
+    _check_dtype(thresholds, torch.float32, "thresholds")
+    bitwidth, N, C, H, W = int(bitwidth), int(N), int(C), int(H), int(W)
+    if bitwidth not in (1, 2):
+        raise RuntimeError(f"bitwidth must be 1 or 2, got {bitwidth}")
+    if min(N, C, H, W) < 1:
+        raise RuntimeError("N, C, H, W must be positive")
+    if X.numel() != N * C * H * W:
+        raise RuntimeError(f"X has {X.numel()} elements, expected N*C*H*W = {N * C * H * W}")
+    if thresholds.numel() < N:
+        raise RuntimeError(f"thresholds has {thresholds.numel()} elements, expected at least N = {N}")
+    if thresholds.device != X.device:
+        raise RuntimeError("X and thresholds must be on the same device")
+    PC = packed_channels(C)
+    with torch.cuda.device(X.device):
+        QX = torch.empty((N, H, W, PC, bitwidth), dtype=torch.int64, device=X.device)
+        BTN = torch.empty((N,), dtype=torch.int32, device=X.device)
+        _capi.check(_lib, _lib.tab_quantize_nchw(X.data_ptr(), thresholds.data_ptr(), bitwidth, N, C, H, W,
+                                                 QX.data_ptr(), BTN.data_ptr(), _stream()))
+    return [QX, BTN]
+
+
 def QuantizeFormat(X, thresholds, type, N, H, W, C):
     """Packer of conv types 4 (DoReFa 2-bit levels; QX int64 (N,H,W,PC,2), plane 0 = weight-2 bit)
     and 5 (RTN 2-bit fields; QX int64 (N,H,W,ceil(C/32))), for activations and weights alike.  The
@@ -248,6 +276,6 @@ def set_conv_kernel(kernel=CONV_AUTO, tile=-1):
 TAB_Quantize = Quantize
 TAB_Conv2d = Conv2d
 
-__all__ = ["Quantize", "QuantizeFormat", "Conv2d", "Conv2dPacked", "Conv2dPackedOut", "Threshold", "TAB_Quantize", "TAB_Conv2d", "TabError",
+__all__ = ["Quantize", "QuantizeNCHW", "QuantizeFormat", "Conv2d", "Conv2dPacked", "Conv2dPackedOut", "Threshold", "TAB_Quantize", "TAB_Conv2d", "TabError",
            "packed_channels", "out_shape", "version", "TNN", "TBN", "BTN", "BNN", "set_conv_kernel",
            "CONV_AUTO", "CONV_MATRIX", "CONV_POPCOUNT"]

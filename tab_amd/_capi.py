@@ -19,6 +19,7 @@ SIGNATURES = {
     "tab_operand_words": (_int, [_int] * 3),
     "tab_out_extent": (_int, [_int] * 4),
     "tab_quantize": (_int, [_vp, _vp, _int, _int, _int, _int, _int, _vp, _vp, _vp]),
+    "tab_quantize_nchw": (_int, [_vp, _vp, _int, _int, _int, _int, _int, _vp, _vp, _vp]),
     "tab_quantize_format": (_int, [_vp, _vp, _int, _int, _int, _int, _int, _vp, _vp]),
     "tab_threshold_workspace_bytes": (_sz, [_int, ctypes.c_long]),
     "tab_threshold": (_int, [_vp, _int, ctypes.c_long, ctypes.c_float, _vp, _vp, _sz, _vp]),

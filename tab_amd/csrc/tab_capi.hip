@@ -117,6 +117,20 @@ int tab_quantize(const float *dev_X, const float *dev_ths, int bitwidth, int N, 
     return TAB_OK;
 }
 
+int tab_quantize_nchw(const float *dev_X, const float *dev_ths, int bitwidth, int N, int C, int H, int W,
+                      int64_t *dev_QX, int32_t *dev_BTN, void *stream)
+{
+    if (bitwidth != 1 && bitwidth != 2) return fail(TAB_ERR_BAD_ARGUMENT, "bitwidth must be 1 or 2, got %d", bitwidth);
+    if (N < 1 || H < 1 || W < 1 || C < 1) return fail(TAB_ERR_BAD_ARGUMENT, "N, C, H, W must be positive");
+    if (!dev_X || !dev_ths || !dev_QX || !dev_BTN) return fail(TAB_ERR_BAD_ARGUMENT, "null device pointer");
+    if (N > 65535 || tab_packed_channels(C) > 65535)
+        return fail(TAB_ERR_BAD_SHAPE, "N and ceil(C/64) must be below 65536 (grid dimensions), got %d and %d", N, tab_packed_channels(C));
+    hipError_t e = tab::launch_quantize_nchw(dev_X, dev_ths, bitwidth, N, C, (long)H * W, reinterpret_cast<uint64_t *>(dev_QX),
+                                             dev_BTN, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return device_fail(e, "quantize launch");
+    return TAB_OK;
+}
+
 size_t tab_threshold_workspace_bytes(int N, long per_item)
 {
     if (N < 1 || per_item < 1) return 0;

@@ -68,6 +68,10 @@ hipError_t launch_conv_mfma_rtn(const ConvArgs &args, int shape, hipStream_t str
 hipError_t launch_quantize(const float *x, const float *ths, int bitwidth, long pixels_per_item,
                            long items, int C, uint64_t *qx, int32_t *btn, hipStream_t stream);
 
+// The same quantizer reading x as [N][C][H*W] (the CPU path's input layout, TAB_CPU.cpp:20-206); output as above.
+hipError_t launch_quantize_nchw(const float *x, const float *ths, int bitwidth, int N, int C, long HW, uint64_t *qx,
+                                int32_t *btn, hipStream_t stream);
+
 // Packers of the CPU-only conv types: format 4 = DoReFa 2-bit levels, 5 = RTN fields.
 hipError_t launch_quantize_format(const float *x, const float *ths, int format, long pixels_per_item, long items, int C,
                                   uint64_t *qx, hipStream_t stream);

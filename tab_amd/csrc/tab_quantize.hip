@@ -270,6 +270,69 @@ __global__ __launch_bounds__(kThreads) void quantize_ballot_format(const float *
     }
 }
 
+// The same quantizers on an NCHW tensor, the layout the reference's CPU quantizers read
+// (Parallel_Ternarize_NCHWB_to_NHWCB / Parallel_Binarize_NCHW_to_NHWC, TAB_CPU.cpp:20-206), into the same NHWC
+// packed output.  A thread owns VEC consecutive pixels of one image and one 64-channel word: it walks the
+// word's channels, VEC floats per load (consecutive threads read consecutive pixels of one channel plane,
+// so every load instruction is contiguous), and shifts each compare bit into the words it holds in
+// registers: no cross-lane step at all.  grid = (ceil(H*W / (VEC * 256)), PC, N).
+template <int BITS, int VEC>
+__global__ __launch_bounds__(kThreads) void quantize_nchw(const float *__restrict__ x, const float *__restrict__ ths,
+                                                          uint64_t *__restrict__ q, int C, long HW, int PC)
+{
+    typedef float vec_t __attribute__((ext_vector_type(VEC)));
+    const int pc = blockIdx.y, n = blockIdx.z;
+    const long s0 = ((long)blockIdx.x * kThreads + threadIdx.x) * VEC;
+    if (s0 >= HW) return;
+    const float t = ths[n];
+    const int c0 = pc * kWordBits;
+    const int channels = C - c0 < kWordBits ? C - c0 : kWordBits;
+    const float *src = x + ((long)n * C + c0) * HW + s0;
+    uint64_t sign[VEC], nz[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; e++) sign[e] = nz[e] = 0;
+    constexpr int kInFlight = VEC == 1 ? 32 : 8;  // the one-pixel form serves small, latency-bound tensors
+    for (int j0 = 0; j0 < channels; j0 += kInFlight) {
+        float v[kInFlight][VEC];
+#pragma unroll
+        for (int u = 0; u < kInFlight; u++) {
+            const int j = j0 + u < channels ? j0 + u : channels - 1;  // clamped: the bit is masked below
+            if (VEC == 1) {
+                v[u][0] = __builtin_nontemporal_load(src + (long)j * HW);
+            } else {
+                const vec_t w = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(src + (long)j * HW));
+#pragma unroll
+                for (int e = 0; e < VEC; e++) v[u][e] = w[e];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kInFlight; u++) {
+            const uint64_t bit = j0 + u < channels ? (uint64_t)1 << (j0 + u) : 0;
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+                if (BITS == 2) {
+                    const bool pos = v[u][e] > t;
+                    const bool neg = !pos && (v[u][e] < -t);
+                    if (pos || neg) nz[e] |= bit;
+                    if (neg) sign[e] |= bit;
+                } else {
+                    if (v[u][e] < t) sign[e] |= bit;
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; e++) {
+        const long pixel = (long)n * HW + s0 + e;
+        if (BITS == 2) {
+            q[(pixel * PC + pc) * 2 + 0] = sign[e];
+            q[(pixel * PC + pc) * 2 + 1] = nz[e];
+        } else {
+            q[pixel * PC + pc] = sign[e];
+        }
+    }
+}
+
 __global__ void fill_zero_i32(int32_t *p, long n)
 {
     const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -432,6 +495,35 @@ hipError_t launch_quantize(const float *x, const float *ths, int bitwidth, long 
     if (btn && bitwidth == 2) {
         btn_popcount<<<dim3((unsigned)(items * splits)), dim3(kThreads), 0, stream>>>(
             reinterpret_cast<const ulonglong2 *>(qx), btn, words_per_item, splits);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_quantize_nchw(const float *x, const float *ths, int bitwidth, int N, int C, long HW, uint64_t *qx,
+                                int32_t *btn, hipStream_t stream)
+{
+    const int PC = (C + kWordBits - 1) / kWordBits;
+    const long words_per_item = HW * PC;
+    int splits = 1;
+    if (btn && bitwidth == 2 && N < 512) {
+        while (splits < 64 && (long)N * splits < 512 && words_per_item / (splits * 2) >= 2 * kThreads) splits *= 2;
+    }
+    if (btn && (bitwidth != 2 || splits > 1))
+        fill_zero_i32<<<dim3((unsigned)((N + 255) / 256)), dim3(256), 0, stream>>>(btn, N);
+    // four pixels per thread when the planes allow aligned 16-byte loads and the launch still fills the chip
+    const bool vec4 = HW % 4 == 0 && (uintptr_t)x % 16 == 0 && ((HW + 4 * kThreads - 1) / (4 * kThreads)) * PC * N >= 2048;
+    const long per_block = (vec4 ? 4 : 1) * (long)kThreads;
+    const dim3 grid((unsigned)((HW + per_block - 1) / per_block), (unsigned)PC, (unsigned)N), block(kThreads);
+    if (vec4) {
+        if (bitwidth == 2) quantize_nchw<2, 4><<<grid, block, 0, stream>>>(x, ths, qx, C, HW, PC);
+        else quantize_nchw<1, 4><<<grid, block, 0, stream>>>(x, ths, qx, C, HW, PC);
+    } else {
+        if (bitwidth == 2) quantize_nchw<2, 1><<<grid, block, 0, stream>>>(x, ths, qx, C, HW, PC);
+        else quantize_nchw<1, 1><<<grid, block, 0, stream>>>(x, ths, qx, C, HW, PC);
+    }
+    if (btn && bitwidth == 2) {
+        btn_popcount<<<dim3((unsigned)(N * splits)), dim3(kThreads), 0, stream>>>(reinterpret_cast<const ulonglong2 *>(qx), btn,
+                                                                                 words_per_item, splits);
     }
     return hipGetLastError();
 }

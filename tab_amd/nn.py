@@ -8,7 +8,8 @@ Inference only (the operators have no backward).
 import torch
 from torch import nn
 
-from . import BNN, BTN, TBN, TNN, Conv2d, Conv2dPacked, Conv2dPackedOut, Quantize, Threshold, out_shape
+from . import (BNN, BTN, TBN, TNN, Conv2d, Conv2dPacked, Conv2dPackedOut, Quantize, QuantizeNCHW, Threshold,
+               out_shape)
 
 _ACT_BITS = {TNN: 2, TBN: 2, BTN: 1, BNN: 1}
 _WEIGHT_BITS = {TNN: 2, TBN: 1, BTN: 2, BNN: 1}
@@ -22,8 +23,8 @@ class TABConv2d(nn.Module):
     """2-D convolution with ternary/binary activations and weights.  Holds the packed weights
     (QW) and the BTN popcounts as buffers; the activation threshold is `act_scale * mean|x|` per
     image for ternary activations and 0 for binary ones.  `data_format` is the layout of the
-    input and of the returned tensor: "NCHW" (PyTorch's; converted to the operators' NHWC
-    inside) or "NHWC"."""
+    input and of the returned tensor: "NCHW" (PyTorch's; quantized directly from that layout, the
+    result a permuted view of the operators' NHWC output) or "NHWC"."""
 
     def __init__(self, QW, BTN_W, conv_type, in_channels, out_channels, kernel_size, stride=1, padding=0,
                  act_scale=0.7, data_format="NCHW"):
@@ -51,21 +52,28 @@ class TABConv2d(nn.Module):
         return cls(QW, BTN_W, conv_type, C, KN, (KH, KW), stride, padding, act_scale, data_format)
 
     def forward(self, x):
-        if self.data_format == "NCHW":
+        nchw = self.data_format == "NCHW"
+        if nchw:
             N, C, H, W = x.shape
-            x = x.permute(0, 2, 3, 1)
         else:
             N, H, W, C = x.shape
         if C != self.in_channels:
             raise RuntimeError(f"expected {self.in_channels} input channels, got {C}")
         x = x.to(torch.float32).contiguous()
-        if _ACT_BITS[self.conv_type] == 2:
-            ths = Threshold(x, N, self.act_scale)
+        abits = _ACT_BITS[self.conv_type]
+        if abits == 2:
+            ths = Threshold(x, N, self.act_scale)  # mean|x| per image: the same in either layout
         else:
             ths = torch.zeros(N, dtype=torch.float32, device=x.device)
         (KH, KW), (s1, s2), (p1, p2) = self.kernel_size, self.stride, self.padding
-        y = Conv2d(x, self.QW, ths, self.BTN_W, self.conv_type, p1, p2, s1, s2, N, H, W, C,
-                   self.out_channels, KH, KW)
+        if nchw:
+            # quantized straight from NCHW (no transposed fp32 copy), then the packed entry point
+            QX, _ = QuantizeNCHW(x, ths, abits, N, C, H, W)
+            y = Conv2dPacked(QX, self.QW, self.BTN_W, self.conv_type, p1, p2, s1, s2, N, H, W, C,
+                             self.out_channels, KH, KW)
+        else:
+            y = Conv2d(x, self.QW, ths, self.BTN_W, self.conv_type, p1, p2, s1, s2, N, H, W, C,
+                       self.out_channels, KH, KW)
         OH, OW = out_shape(H, W, KH, KW, p1, p2, s1, s2)
         # the operator's (N,KN,OH,OW)-shaped result is (n,oh,ow,kn) in memory (TAB_GEMM.cu:526)
         y = y.view(N, OH, OW, self.out_channels)
@@ -126,9 +134,9 @@ class TABPackedChain(nn.Module):
         self.data_format = data_format
 
     def forward(self, x):
-        if self.data_format == "NCHW":
+        nchw = self.data_format == "NCHW"
+        if nchw:
             N, C, H, W = x.shape
-            x = x.permute(0, 2, 3, 1)
         else:
             N, H, W, C = x.shape
         first = self.layers[0]
@@ -137,7 +145,7 @@ class TABPackedChain(nn.Module):
         x = x.to(torch.float32).contiguous()
         bits = _ACT_BITS[first.conv_type]
         ths = Threshold(x, N, first.act_scale) if bits == 2 else torch.zeros(N, dtype=torch.float32, device=x.device)
-        q, _ = Quantize(x, ths, bits, N, H, W, C)
+        q, _ = QuantizeNCHW(x, ths, bits, N, C, H, W) if nchw else Quantize(x, ths, bits, N, H, W, C)
         for i, layer in enumerate(self.layers):
             (KH, KW), (s1, s2), (p1, p2) = layer.kernel_size, layer.stride, layer.padding
             args = (layer.conv_type, p1, p2, s1, s2, N, H, W, layer.in_channels, layer.out_channels, KH, KW)

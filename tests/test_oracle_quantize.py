@@ -134,6 +134,18 @@ def test_binary_sign_against_reference_cpu_golden():
     assert np.array_equal(_nhwc_padded(q, p1, p2)[..., 0], g["bin_c128_q"])
 
 
+@pytest.mark.parametrize("name,bits", [("ter_c70", 2), ("ter_c128", 2), ("bin_c128", 1)])
+def test_nchw_reading_against_reference_cpu_golden(name, bits):
+    """quantize_nchw reads [C][H][W] the way the reference's CPU quantizers do (TAB_CPU.cpp:20-206): their
+    committed outputs, interior of the padded buffer."""
+    g = np.load(os.path.join(GOLD, "ref_golden.npz"))
+    C, H, W, p1, p2 = (int(v) for v in g[name + "_dims"])
+    ths = g[name + "_th"] if bits == 2 else [0.0]
+    q, _ = oracle.quantize_nchw(g[name + "_x_chw"], ths, bits, 1, C, H, W)
+    want = g[name + "_q"] if bits == 2 else g[name + "_q"][..., None]
+    assert np.array_equal(_nhwc_padded(q, p1, p2), want)
+
+
 @pytest.mark.skipif(not oracle.have_ref(), reason="oracle/_ref not built (no reference tree)")
 def test_ternary_against_reference_cpu_live():
     rng = np.random.default_rng(11)
