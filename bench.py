@@ -392,6 +392,11 @@ def main():
             quant[f"bitwidth{bitwidth}"] = {"us": round(ms * 1e3, 1), "GBps": round(nbytes / ms / 1e6, 1),
                                             "frac_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
                                             "bytes": nbytes}
+            # the same values read as NCHW (256x256x56x56): the quantizer of PyTorch-layout callers
+            xn = xq.view(qN, qC, qH, qW)
+            ms = event_time_ms(torch, lambda: tab.QuantizeNCHW(xn, ths, bitwidth, qN, qC, qH, qW), 20)
+            quant[f"nchw_bitwidth{bitwidth}"] = {"us": round(ms * 1e3, 1), "GBps": round(nbytes / ms / 1e6, 1),
+                                                 "frac_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
         ms = event_time_ms(torch, lambda: tab.Threshold(xq, qN, 0.7), 20)
         quant["threshold_abs_mean"] = {"us": round(ms * 1e3, 1), "GBps": round(4 * qN * qH * qW * qC / ms / 1e6, 1),
                                        "frac_hbm_peak": round(4 * qN * qH * qW * qC / ms / 1e6 / HBM_PEAK_GBS, 4)}
