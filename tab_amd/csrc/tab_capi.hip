@@ -123,8 +123,8 @@ int tab_quantize_nchw(const float *dev_X, const float *dev_ths, int bitwidth, in
     if (bitwidth != 1 && bitwidth != 2) return fail(TAB_ERR_BAD_ARGUMENT, "bitwidth must be 1 or 2, got %d", bitwidth);
     if (N < 1 || H < 1 || W < 1 || C < 1) return fail(TAB_ERR_BAD_ARGUMENT, "N, C, H, W must be positive");
     if (!dev_X || !dev_ths || !dev_QX || !dev_BTN) return fail(TAB_ERR_BAD_ARGUMENT, "null device pointer");
-    if (N > 65535 || tab_packed_channels(C) > 65535)
-        return fail(TAB_ERR_BAD_SHAPE, "N and ceil(C/64) must be below 65536 (grid dimensions), got %d and %d", N, tab_packed_channels(C));
+    if (((long)N * H * W + 255) / 256 * tab_packed_channels(C) > kMaxIndex)
+        return fail(TAB_ERR_BAD_SHAPE, "tensor too large for one launch (N*H*W/256 * ceil(C/64) workgroups)");
     hipError_t e = tab::launch_quantize_nchw(dev_X, dev_ths, bitwidth, N, C, (long)H * W, reinterpret_cast<uint64_t *>(dev_QX),
                                              dev_BTN, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return device_fail(e, "quantize launch");

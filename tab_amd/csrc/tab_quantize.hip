@@ -275,19 +275,23 @@ __global__ __launch_bounds__(kThreads) void quantize_ballot_format(const float *
 // packed output.  A thread owns VEC consecutive pixels of one image and one 64-channel word: it walks the
 // word's channels, VEC floats per load (consecutive threads read consecutive pixels of one channel plane,
 // so every load instruction is contiguous), and shifts each compare bit into the words it holds in
-// registers: no cross-lane step at all.  grid = (ceil(H*W / (VEC * 256)), PC, N).
+// registers: no cross-lane step at all.  Pixels are numbered through all images (VEC divides H*W, so a
+// thread's pixels share an image), which keeps every workgroup full whatever H*W is.
+// grid = ceil(N*H*W / (VEC * 256)) * PC workgroups, the word index fastest: the workgroups that write the PC
+// words of the same pixels run side by side, so their 8- or 16-byte stores meet in L2 as whole lines.
 template <int BITS, int VEC>
 __global__ __launch_bounds__(kThreads) void quantize_nchw(const float *__restrict__ x, const float *__restrict__ ths,
-                                                          uint64_t *__restrict__ q, int C, long HW, int PC)
+                                                          uint64_t *__restrict__ q, int N, int C, long HW, int PC)
 {
     typedef float vec_t __attribute__((ext_vector_type(VEC)));
-    const int pc = blockIdx.y, n = blockIdx.z;
-    const long s0 = ((long)blockIdx.x * kThreads + threadIdx.x) * VEC;
-    if (s0 >= HW) return;
+    const int pc = blockIdx.x % PC;
+    const long g0 = ((long)(blockIdx.x / PC) * kThreads + threadIdx.x) * VEC;  // first pixel, counted through all images
+    if (g0 >= (long)N * HW) return;
+    const long n = g0 / HW, s0 = g0 - n * HW;
     const float t = ths[n];
     const int c0 = pc * kWordBits;
     const int channels = C - c0 < kWordBits ? C - c0 : kWordBits;
-    const float *src = x + ((long)n * C + c0) * HW + s0;
+    const float *src = x + (n * C + c0) * HW + s0;
     uint64_t sign[VEC], nz[VEC];
 #pragma unroll
     for (int e = 0; e < VEC; e++) sign[e] = nz[e] = 0;
@@ -323,7 +327,7 @@ __global__ __launch_bounds__(kThreads) void quantize_nchw(const float *__restric
     }
 #pragma unroll
     for (int e = 0; e < VEC; e++) {
-        const long pixel = (long)n * HW + s0 + e;
+        const long pixel = g0 + e;
         if (BITS == 2) {
             q[(pixel * PC + pc) * 2 + 0] = sign[e];
             q[(pixel * PC + pc) * 2 + 1] = nz[e];
@@ -511,15 +515,18 @@ hipError_t launch_quantize_nchw(const float *x, const float *ths, int bitwidth, 
     if (btn && (bitwidth != 2 || splits > 1))
         fill_zero_i32<<<dim3((unsigned)((N + 255) / 256)), dim3(256), 0, stream>>>(btn, N);
     // four pixels per thread when the planes allow aligned 16-byte loads and the launch still fills the chip
-    const bool vec4 = HW % 4 == 0 && (uintptr_t)x % 16 == 0 && ((HW + 4 * kThreads - 1) / (4 * kThreads)) * PC * N >= 2048;
+    const long pixels = (long)N * HW;
+    const bool vec4 = HW % 4 == 0 && (uintptr_t)x % 16 == 0 && ((pixels + 4 * kThreads - 1) / (4 * kThreads)) * PC >= 2048;
     const long per_block = (vec4 ? 4 : 1) * (long)kThreads;
-    const dim3 grid((unsigned)((HW + per_block - 1) / per_block), (unsigned)PC, (unsigned)N), block(kThreads);
+    const long blocks = (pixels + per_block - 1) / per_block;
+    if (blocks * PC > 0x7fffffffL) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)(blocks * PC)), block(kThreads);
     if (vec4) {
-        if (bitwidth == 2) quantize_nchw<2, 4><<<grid, block, 0, stream>>>(x, ths, qx, C, HW, PC);
-        else quantize_nchw<1, 4><<<grid, block, 0, stream>>>(x, ths, qx, C, HW, PC);
+        if (bitwidth == 2) quantize_nchw<2, 4><<<grid, block, 0, stream>>>(x, ths, qx, N, C, HW, PC);
+        else quantize_nchw<1, 4><<<grid, block, 0, stream>>>(x, ths, qx, N, C, HW, PC);
     } else {
-        if (bitwidth == 2) quantize_nchw<2, 1><<<grid, block, 0, stream>>>(x, ths, qx, C, HW, PC);
-        else quantize_nchw<1, 1><<<grid, block, 0, stream>>>(x, ths, qx, C, HW, PC);
+        if (bitwidth == 2) quantize_nchw<2, 1><<<grid, block, 0, stream>>>(x, ths, qx, N, C, HW, PC);
+        else quantize_nchw<1, 1><<<grid, block, 0, stream>>>(x, ths, qx, N, C, HW, PC);
     }
     if (btn && bitwidth == 2) {
         btn_popcount<<<dim3((unsigned)(N * splits)), dim3(kThreads), 0, stream>>>(reinterpret_cast<const ulonglong2 *>(qx), btn,

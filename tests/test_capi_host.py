@@ -86,7 +86,7 @@ def test_c_abi_rejects_bad_arguments_without_launching():
     assert b"exact accumulation" in lib.tab_last_error()
     assert lib.tab_conv2d_packed(p, p, p, 5, 0, 0, 1, 1, 1, 4, 4, 32 * 65536, 4, 1, 1, p, None) == -2
     assert lib.tab_quantize_nchw(p, p, 3, 1, 64, 1, 1, p, p, None) == -1 and b"bitwidth" in lib.tab_last_error()
-    assert lib.tab_quantize_nchw(p, p, 2, 70000, 64, 1, 1, p, p, None) == -2
+    assert lib.tab_quantize_nchw(p, p, 2, 60000, 64 * 100, 1000, 1000, p, p, None) == -2
     assert lib.tab_quantize_nchw(p, p, 2, 1, 64, 1, 1, None, p, None) == -1
     assert lib.tab_quantize_format(p, p, 3, 1, 1, 1, 64, p, None) == -1 and b"4 (DRF) or 5 (RTN)" in lib.tab_last_error()
     assert lib.tab_quantize_format(p, None, 4, 1, 1, 1, 64, p, None) == -1
