@@ -7,8 +7,11 @@
 // of a one-plane activation granule must lie in one filter tap, so PC is even; a chunk may span taps
 // (each wave instruction decodes the tap of its granules, one scalar computation).
 // An LDS-direct load writes lane i's 16 bytes at base + 16*i, and a lane whose offset is out of
-// range writes zeros (padding taps, rows past M, filters past KN), so granule index = piece * ROWS +
-// row with one wave instruction covering 64 consecutive rows of one piece.
+// range writes zeros (padding taps, rows past M, filters past KN).  The P granules of a row and chunk are
+// taken in runs of RUN = 4, 2 or 1 (see granule_run): granule index = (run * ROWS + row) * RUN +
+// column, so RUN neighbouring lanes fetch 16 * RUN contiguous bytes of one row and a wave instruction touches
+// 64 / RUN cache lines, and column = (granule of the run + swizzle(row)) % RUN spreads the 16-byte reads of one
+// granule of 16 consecutive rows over the LDS banks.  A run of an activation row must lie within one filter tap.
 //
 // Per pair of words p the half-waves take alternate words: lane (kb, r) owns word 2p + kb of row r and
 // multiplies its low half in one MFMA and its high half in the next.  A one-plane operand reads its
@@ -29,6 +32,20 @@ __device__ __forceinline__ void load16_to_lds(__amdgpu_buffer_rsrc_t rsrc, uint3
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void *)dst, 16, byte_offset, 0, 0, 0);
 }
 
+// Granules of a row and chunk fetched by neighbouring lanes.
+// (Pairs of one-plane granules, read 8 bytes a lane, measured no faster than single ones.)
+constexpr int granule_run(int per_row, int planes) { return per_row % 4 == 0 ? 4 : (per_row % 2 == 0 && planes == 2 ? 2 : 1); }
+
+// Column rotation of a row (mod 16) in a run layout.  Reads of one granule by 16 consecutive rows must fall into 16
+// different 16-byte bank groups, by 8 consecutive rows into 8 different ones: with RUN = 4 the rotation differs
+// between rows r, r+4, r+8, r+12 and between the four row pairs of an aligned 8; with RUN = 2 between r and r+4
+// within an aligned 8 and between r and r+8.
+template <int RUN>
+__device__ __forceinline__ int run_swizzle(int row)
+{
+    return RUN == 4 ? ((row >> 1) + (row >> 3)) & 3 : (RUN == 2 ? ((row >> 2) + (row >> 3)) & 1 : 0);
+}
+
 template <int TYPE, int WM, int WN, int TM, int TN, int KCH>
 __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM * TN > 4 ? 2 : (WM * TM > 4 ? 3 : 4)))) void conv_mfma_direct(const ConvArgs p)
 {
@@ -40,6 +57,7 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
     constexpr int A_GRANULES = PA * BM, B_GRANULES = PB * BN;
     constexpr int A_ITEMS = (A_GRANULES + kConvThreads - 1) / kConvThreads, B_ITEMS = (B_GRANULES + kConvThreads - 1) / kConvThreads;
     constexpr int BUF_DWORDS = 4 * (A_ITEMS + B_ITEMS) * kConvThreads;  // whole wave instructions
+    constexpr int A_RUN = granule_run(PA, APL), B_RUN = granule_run(PB, BPL);
 
     __shared__ __attribute__((aligned(16))) uint32_t lds[2 * BUF_DWORDS];
 
@@ -50,7 +68,7 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
     const int tile_m = blockIdx.x % p.tiles_m, tile_n = blockIdx.x / p.tiles_m;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
-    // ---- what this lane fetches: granule idx = tid + i * 256 = piece * ROWS + row -------------------
+    // ---- what this lane fetches: granule idx = tid + i * 256 = (run * ROWS + row) * RUN + column ------
     const int pixels = p.OH * p.OW;
     const int n_first = m0 / pixels;  // uniform
     const size_t image_words = (size_t)p.H * p.W * p.PC * APL;
@@ -62,7 +80,9 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
 #pragma unroll
     for (int i = 0; i < A_ITEMS; i++) {
         const int idx = tid + i * kConvThreads;
-        const int piece = idx / BM, row = idx % BM;
+        const int row = idx / A_RUN % BM;
+        const int in_run = (idx % A_RUN - run_swizzle<A_RUN>(row & 15)) & (A_RUN - 1);
+        const int piece = idx / A_RUN / BM * A_RUN + in_run;
         const int a_m = m0 + row;
         const bool live = piece < PA && a_m < p.M;
         const int mm = live ? a_m : m0;
@@ -71,7 +91,8 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
         const int oh = rem / p.OW, ow = rem - oh * p.OW;
         ih0[i] = live ? oh * p.s1 - p.p1 : -(1 << 30);  // a dead granule fails every bounds check
         iw0[i] = ow * p.s2 - p.p2;
-        a_base[i] = (uint32_t)((((n - n_first) * p.H + (oh * p.s1 - p.p1)) * p.W + iw0[i]) * p.PC) * (uint32_t)(APL * 8);
+        a_base[i] = (uint32_t)((((n - n_first) * p.H + (oh * p.s1 - p.p1)) * p.W + iw0[i]) * p.PC) * (uint32_t)(APL * 8) +
+                    (uint32_t)in_run * 16u;
     }
     const size_t filter_bytes = (size_t)p.G * BPL * 8;
     const size_t b_bytes = (size_t)(p.KN - n0) * filter_bytes;
@@ -80,7 +101,8 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
 #pragma unroll
     for (int i = 0; i < B_ITEMS; i++) {
         const int idx = tid + i * kConvThreads;
-        const int piece = idx / BN, row = idx % BN;
+        const int row = idx / B_RUN % BN;
+        const int piece = idx / B_RUN / BN * B_RUN + ((idx % B_RUN - run_swizzle<B_RUN>(row & 15)) & (B_RUN - 1));
         const bool live = piece < PB && (n0 + row) < p.KN;
         b_base[i] = live ? (uint32_t)row * (uint32_t)filter_bytes + (uint32_t)piece * 16u : kNoFilter;
     }
@@ -90,8 +112,8 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
         const int g0 = chunk * KCH;  // first word of the chunk
 #pragma unroll
         for (int i = 0; i < A_ITEMS; i++) {
-            // the granule's first word and its tap: the same for the 64 rows this wave instruction moves
-            const int g = g0 + (i * kConvThreads + wave * 64) / BM * (APL == 1 ? 2 : 1);
+            // the first word of the run this wave instruction moves and its tap: the same for all its rows
+            const int g = g0 + (i * kConvThreads + wave * 64) / A_RUN / BM * A_RUN * (APL == 1 ? 2 : 1);
             const uint32_t tap = fastdiv((uint32_t)g, p.div_pc);
             const int pc = g - (int)tap * p.PC;
             const int kh = (int)fastdiv(tap, p.div_kw);
@@ -125,12 +147,19 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
 
-    // dword offset of this lane's part of granule (pair 0, its row): one-plane: 8 bytes of the pair's granule;
-    // two-plane: the granule of its own word
+    // dword offset of this lane's part of a pair of words: one-plane: 8 bytes of the pair's granule; two-plane:
+    // the granule of its own word, 2 * pair + kb.  Tile and wave offsets are multiples of 32 rows, so the
+    // column rotation is that of r.
     const int a_row = wm * (32 * TM) + r, b_row = wn * (32 * TN) + r;
-    constexpr int A_PAIR = (APL == 1 ? 1 : 2) * BM * 4, B_PAIR = (BPL == 1 ? 1 : 2) * BN * 4;  // dwords between pairs
-    const int a_off = (APL == 1 ? 4 * a_row + 2 * kb : 4 * (kb * BM + a_row));
-    const int b_off = 4 * A_ITEMS * kConvThreads + (BPL == 1 ? 4 * b_row + 2 * kb : 4 * (kb * BN + b_row));
+    const int a_sw = run_swizzle<A_RUN>(r & 15), b_sw = run_swizzle<B_RUN>(r & 15);
+    auto lane_part = [kb](int planes, int run, int rows, int row, int sw, int pair) {
+        const int granule = planes == 1 ? pair : 2 * pair + kb;
+        // granule / run and granule % run without dividing by what the compiler cannot see is 0 or 1
+        const int group = run == 1 ? granule : (planes == 1 ? pair / run : 2 * pair / run);
+        const int in_run = run == 1 ? 0 : (planes == 1 ? pair % run : 2 * pair % run + kb);
+        return ((group * rows + row) * run + ((in_run + sw) & (run - 1))) * 4 + (planes == 1 ? 2 * kb : 0);
+    };
+    constexpr int B_REGION = 4 * A_ITEMS * kConvThreads;
 
     for (int chunk = 0; chunk < p.nchunks; chunk++) {
         const bool more = chunk + 1 < p.nchunks;
@@ -141,7 +170,7 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
         auto read_pair = [&](int pair) {
 #pragma unroll
             for (int mt = 0; mt < TM; mt++) {
-                const uint32_t *src = buf + a_off + pair * A_PAIR + mt * 32 * 4;
+                const uint32_t *src = buf + lane_part(APL, A_RUN, BM, a_row, a_sw, pair) + mt * 32 * A_RUN * 4;
                 if (APL == 1) {
                     const u32x2 v = *reinterpret_cast<const u32x2 *>(src);
                     a_w[pair & 1][mt][0] = v[0]; a_w[pair & 1][mt][1] = v[1];
@@ -153,7 +182,7 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
             }
 #pragma unroll
             for (int nt = 0; nt < TN; nt++) {
-                const uint32_t *src = buf + b_off + pair * B_PAIR + nt * 32 * 4;
+                const uint32_t *src = buf + B_REGION + lane_part(BPL, B_RUN, BN, b_row, b_sw, pair) + nt * 32 * B_RUN * 4;
                 if (BPL == 1) {
                     const u32x2 v = *reinterpret_cast<const u32x2 *>(src);
                     b_w[pair & 1][nt][0] = v[0]; b_w[pair & 1][nt][1] = v[1];
@@ -206,7 +235,9 @@ template <int TYPE, int WM, int WN, int TM, int TN, int KCH>
 hipError_t launch_mfma_direct(ConvArgs a, hipStream_t stream)
 {
     constexpr int BM = 32 * WM * TM, BN = 32 * WN * TN;
-    if (a.G % KCH != 0 || (Planes<TYPE>::A == 1 && a.PC % 2 != 0)) return hipErrorInvalidValue;
+    // words of a run of activation granules, which must not straddle filter taps
+    constexpr int A_RUN_WORDS = granule_run(KCH * Planes<TYPE>::A / 2, Planes<TYPE>::A) * (Planes<TYPE>::A == 1 ? 2 : 1);
+    if (a.G % KCH != 0 || a.PC % A_RUN_WORDS != 0) return hipErrorInvalidValue;
     a.kcw = KCH;
     a.nchunks = a.G / KCH;
     a.tiles_m = (a.M + BM - 1) / BM;
