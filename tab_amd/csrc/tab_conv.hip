@@ -362,8 +362,13 @@ int conv_mfma_shape(int conv_type, const ConvArgs &a)
     // short K: the per-tile prologue and epilogue weigh more, so a shape needs more tiles to pay
     const long enough = a.G >= 72 ? 192 : (a.G >= 36 ? 300 : 1024);
     // eight tiles per wave share each expanded operand between more MFMAs (the dearer operand gets the
-    // 4-tile side): +2-18 %, but only when the launch is many rounds of these big tiles
-    if (a.G >= 36 && tiles(256, 128) >= 2560) {
+    // 4-tile side): +2-18 %, but only when the launch is many rounds of these big tiles (512 run at a time), or,
+    // with long K and a two-plane operand (3-10 %), at least two rounds or most of a single one; in between the
+    // tail of the last round costs more than the shape gains
+    const long big_tiles = tiles(256, 128);
+    const bool rounds = a.G >= 36 && big_tiles >= 2560;
+    const bool long_k = type != 3 && a.G >= 72 && (big_tiles >= 1024 || (big_tiles >= 384 && big_tiles <= 512));
+    if (rounds || long_k) {
         if (type == 1 && a.KN >= 256) return 6;
         if (type != 1 && a.KN >= 128) return 5;
     }
