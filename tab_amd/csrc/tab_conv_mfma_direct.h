@@ -10,7 +10,7 @@
 // range writes zeros (padding taps, rows past M, filters past KN).  The P granules of a row and chunk are
 // taken in runs of RUN = 4, 2 or 1 (see granule_run): granule index = (run * ROWS + row) * RUN +
 // column, so RUN neighbouring lanes fetch 16 * RUN contiguous bytes of one row and a wave instruction touches
-// 64 / RUN cache lines, and column = (granule of the run + swizzle(row)) % RUN spreads the 16-byte reads of one
+// 64 / RUN cache lines, and column = (granule of the run + run_swizzle(row)) % RUN spreads the 16-byte reads of one
 // granule of 16 consecutive rows over the LDS banks.  A run of an activation row must lie within one filter tap.
 //
 // Per pair of words p the half-waves take alternate words: lane (kb, r) owns word 2p + kb of row r and
@@ -82,9 +82,9 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
         const int idx = tid + i * kConvThreads;
         const int row = idx / A_RUN % BM;
         const int in_run = (idx % A_RUN - run_swizzle<A_RUN>(row & 15)) & (A_RUN - 1);
-        const int piece = idx / A_RUN / BM * A_RUN + in_run;
+        const int granule = idx / A_RUN / BM * A_RUN + in_run;  // of the row's chunk
         const int a_m = m0 + row;
-        const bool live = piece < PA && a_m < p.M;
+        const bool live = granule < PA && a_m < p.M;
         const int mm = live ? a_m : m0;
         const int n = mm / pixels;
         const int rem = mm - n * pixels;
@@ -102,12 +102,12 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
     for (int i = 0; i < B_ITEMS; i++) {
         const int idx = tid + i * kConvThreads;
         const int row = idx / B_RUN % BN;
-        const int piece = idx / B_RUN / BN * B_RUN + ((idx % B_RUN - run_swizzle<B_RUN>(row & 15)) & (B_RUN - 1));
-        const bool live = piece < PB && (n0 + row) < p.KN;
-        b_base[i] = live ? (uint32_t)row * (uint32_t)filter_bytes + (uint32_t)piece * 16u : kNoFilter;
+        const int granule = idx / B_RUN / BN * B_RUN + ((idx % B_RUN - run_swizzle<B_RUN>(row & 15)) & (B_RUN - 1));
+        const bool live = granule < PB && (n0 + row) < p.KN;
+        b_base[i] = live ? (uint32_t)row * (uint32_t)filter_bytes + (uint32_t)granule * 16u : kNoFilter;
     }
 
-    static_assert(BM % 64 == 0 && BN % 64 == 0, "one wave instruction moves 64 rows of one piece");
+    static_assert(BM % 64 == 0 && BN % 64 == 0, "one wave instruction moves 64 / RUN rows of one run");
     auto fetch = [&](int chunk, uint32_t *buf) {
         const int g0 = chunk * KCH;  // first word of the chunk
 #pragma unroll
