@@ -115,7 +115,7 @@ __global__ __launch_bounds__(kThreads) void quantize_rows64(const floatx4 *__res
                                                             long rows_per_item)
 {
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: so are row0 and the item test below
     const int sub = lane >> 4;  // which of the 4 rows of a load
     const int l = lane & 15;    // float4 within the row
     const long row0 = ((long)blockIdx.x * kWavesPerBlock + wave) * (4 * LOADS);
@@ -127,18 +127,16 @@ __global__ __launch_bounds__(kThreads) void quantize_rows64(const floatx4 *__res
 #pragma unroll
     for (int u = 0; u < LOADS; u++) {
         const long r = row0 + u * 4 + sub;
-        v[u] = (r < rows) ? __builtin_nontemporal_load(&x[r * 16 + l]) : floatx4{0.f, 0.f, 0.f, 0.f};
+        // rows past the end read the last row again (not stored): straight-line loads, no branch per load
+        v[u] = __builtin_nontemporal_load(&x[(r < rows ? r : rows - 1) * 16 + l]);
     }
 
     const long item_first = row0 / rows_per_item;
     const bool one_item = (row_last / rows_per_item) == item_first;  // wave-uniform
     const float t_first = ths[item_first];
 
-#pragma unroll
-    for (int u = 0; u < LOADS; u++) {
+    auto finish = [&](int u, float t) {
         const long r = row0 + u * 4 + sub;
-        float t = t_first;
-        if (!one_item) t = ths[(r < rows ? r : rows - 1) / rows_per_item];
         uint32_t sign, nz, out[4];
         compare4<BITS>(v[u], t, sign, nz);
         pack_row<BITS>(sign, nz, l, out);  // lane 0 stores the whole element (8 or 16 bytes) at once
@@ -146,6 +144,18 @@ __global__ __launch_bounds__(kThreads) void quantize_rows64(const floatx4 *__res
             if (r < rows && l == 0) *reinterpret_cast<uintx4 *>(q + r * 4) = uintx4{out[0], out[1], out[2], out[3]};
         } else {
             if (r < rows && l == 0) *reinterpret_cast<uintx2 *>(q + r * 2) = uintx2{out[0], out[1]};
+        }
+    };
+    // two copies of the loop under a scalar branch: the common one has no load but x in flight, so each load is
+    // waited for on its own
+    if (one_item) {
+#pragma unroll
+        for (int u = 0; u < LOADS; u++) finish(u, t_first);
+    } else {
+#pragma unroll
+        for (int u = 0; u < LOADS; u++) {
+            const long r = row0 + u * 4 + sub;
+            finish(u, ths[(r < rows ? r : rows - 1) / rows_per_item]);
         }
     }
 }
@@ -171,10 +181,10 @@ __global__ __launch_bounds__(64) void quantize_rows64_strided(const floatx4 *__r
     floatx4 v[LOADS];
 #pragma unroll
     for (int u = 0; u < LOADS; u++) {
-        const int j = j0 + u * 4 + sub;
+        const int j = min(j0 + u * 4 + sub, line_words - 1);  // words past the line read its last word again (not stored)
         const int ow = (int)fastdiv((uint32_t)j, div_pc), pc = j - ow * PC;
         const long r = (in_line + (long)ow * s2) * PC + pc;
-        v[u] = (j < line_words) ? __builtin_nontemporal_load(&x[r * 16 + l]) : floatx4{0.f, 0.f, 0.f, 0.f};
+        v[u] = __builtin_nontemporal_load(&x[r * 16 + l]);
     }
 #pragma unroll
     for (int u = 0; u < LOADS; u++) {
