@@ -306,7 +306,7 @@ __global__ __launch_bounds__(kThreads) void quantize_nchw(const float *__restric
 #pragma unroll
     for (int e = 0; e < VEC; e++) sign[e] = nz[e] = 0;
     constexpr int kInFlight = VEC == 1 ? 32 : 8;  // the one-pixel form serves small, latency-bound tensors
-    for (int j0 = 0; j0 < channels; j0 += kInFlight) {
+    auto step = [&](const int j0) {
         float v[kInFlight][VEC];
 #pragma unroll
         for (int u = 0; u < kInFlight; u++) {
@@ -334,6 +334,12 @@ __global__ __launch_bounds__(kThreads) void quantize_nchw(const float *__restric
                 }
             }
         }
+    };
+    if (channels == kWordBits) {  // a whole word: unrolled, every bit position a constant
+#pragma unroll
+        for (int j0 = 0; j0 < kWordBits; j0 += kInFlight) step(j0);
+    } else {
+        for (int j0 = 0; j0 < channels; j0 += kInFlight) step(j0);
     }
 #pragma unroll
     for (int e = 0; e < VEC; e++) {
