@@ -201,7 +201,99 @@ __global__ __launch_bounds__(64) void quantize_rows64_strided(const floatx4 *__r
     }
 }
 
-// General path (any C, any alignment): one wave per (pixel, word); lane i tests channel
+// OR over the LP lanes (a power of two up to 16, aligned inside a DPP row) of a group; every lane gets the result.
+template <int LP>
+__device__ __forceinline__ uint32_t or_reduce_group(uint32_t v)
+{
+    if (LP >= 2) v |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, true);    // quad_perm [1,0,3,2]
+    if (LP >= 4) v |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xF, 0xF, true);    // quad_perm [2,3,0,1]
+    if (LP >= 8) v |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xF, 0xF, true);   // row_half_mirror
+    if (LP >= 16) v |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x140, 0xF, 0xF, true);  // row_mirror
+    return v;
+}
+
+// General path (any C, any alignment of x; pixels * PC < 2^31): a group of LP lanes takes one (pixel, word) row of
+// up to 4 * LP channels, lane l the channels l, l + LP, l + 2 LP, l + 3 LP of the word (so a wave-wide load reads
+// runs of 4 * LP bytes, and neighbouring groups neighbouring rows); LP = 16 serves words of up to 64 channels,
+// smaller groups tensors of few channels (LP = 1: a lane per pixel).  Eight rows per group are in flight.  The
+// lanes' compare bits are ORed over the group; unused high bits of a tail word stay 0 (TAB_GEMM.cu:203-206).
+template <int BITS, int LP>
+__global__ __launch_bounds__(kThreads) void quantize_groups(const float *__restrict__ x, const float *__restrict__ ths,
+                                                            uint32_t *__restrict__ q, long rows, long pixels_per_item,
+                                                            int C, int PC)
+{
+    constexpr int GROUPS = 64 / LP;  // rows per wave-wide load
+    constexpr int U = 8;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int group = lane / LP, l = lane % LP;
+    const long row0 = ((long)blockIdx.x * kWavesPerBlock + wave) * (GROUPS * U);
+    if (row0 >= rows) return;
+    long row_last = row0 + GROUPS * U - 1;
+    if (row_last > rows - 1) row_last = rows - 1;
+
+    float v[U][4];
+    int channels[U];  // of the row's word
+    long pixel[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const long r = row0 + u * GROUPS + group;
+        const uint32_t rc = (uint32_t)(r < rows ? r : rows - 1);  // rows past the end read the last row again (not stored)
+        const uint32_t px = PC == 1 ? rc : rc / (uint32_t)PC;
+        const int c0 = (int)(rc - px * (uint32_t)PC) * kWordBits;
+        channels[u] = C - c0 < kWordBits ? C - c0 : kWordBits;
+        pixel[u] = px;
+        const float *src = x + (long)px * C + c0;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int ch = l + LP * e;  // past the word: its last channel again, masked below
+            v[u][e] = __builtin_nontemporal_load(src + (ch < channels[u] ? ch : channels[u] - 1));
+        }
+    }
+
+    const long item_first = (row0 / PC) / pixels_per_item;
+    const bool one_item = ((row_last / PC) / pixels_per_item) == item_first;  // scalar
+    const float t_first = ths[item_first];
+
+    auto finish = [&](int u, float t) {
+        uint32_t w[4] = {0, 0, 0, 0};  // sign low, sign high, nonzero low, nonzero high
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int ch = l + LP * e;
+            const bool valid = ch < channels[u];
+            const int half = LP * e >= 32 ? 1 : 0;             // LP * e is 0, 16, 32, 48 when channels reach 32
+            const int shift = l + (LP * e - 32 * half);
+            if (BITS == 2) {
+                const bool pos = v[u][e] > t;
+                const bool neg = !pos && (v[u][e] < -t);
+                w[half] |= (uint32_t)(valid && neg) << shift;
+                w[2 + half] |= (uint32_t)(valid && (pos || neg)) << shift;
+            } else {
+                w[half] |= (uint32_t)(valid && (v[u][e] < t)) << shift;
+            }
+        }
+        const long r = row0 + u * GROUPS + group;
+        const uint32_t s_lo = or_reduce_group<LP>(w[0]), s_hi = LP == 16 ? or_reduce_group<LP>(w[1]) : 0u;
+        if (BITS == 2) {
+            const uint32_t n_lo = or_reduce_group<LP>(w[2]), n_hi = LP == 16 ? or_reduce_group<LP>(w[3]) : 0u;
+            if (r < rows && l == 0) {  // QX is aligned to its 8-byte words only
+                *reinterpret_cast<uintx2 *>(q + r * 4) = uintx2{s_lo, s_hi};
+                *reinterpret_cast<uintx2 *>(q + r * 4 + 2) = uintx2{n_lo, n_hi};
+            }
+        } else {
+            if (r < rows && l == 0) *reinterpret_cast<uintx2 *>(q + r * 2) = uintx2{s_lo, s_hi};
+        }
+    };
+    if (one_item) {
+#pragma unroll
+        for (int u = 0; u < U; u++) finish(u, t_first);
+    } else {
+#pragma unroll
+        for (int u = 0; u < U; u++) finish(u, ths[pixel[u] / pixels_per_item]);
+    }
+}
+
+// Fallback of the general path for tensors of 2^31 rows or more: one wave per (pixel, word); lane i tests channel
 // word*64 + i and the two wave-wide ballots are the packed words, LSB first
 // (onebit[i] = 1 << i, TAB_GEMM.cu:252-258).  Unused high bits of a tail word stay 0
 // (TAB_GEMM.cu:203-206).
@@ -462,6 +554,30 @@ hipError_t launch_threshold(const float *x, long items, long per_item, float sca
     return hipGetLastError();
 }
 
+template <int LP>
+void launch_quantize_groups_of(const float *x, const float *ths, int bitwidth, long rows, long pixels_per_item, int C, int PC,
+                               uint32_t *q, hipStream_t stream)
+{
+    const long per_block = (long)kWavesPerBlock * (64 / LP) * 8;
+    const dim3 grid((unsigned)((rows + per_block - 1) / per_block)), block(kThreads);
+    if (bitwidth == 2)
+        quantize_groups<2, LP><<<grid, block, 0, stream>>>(x, ths, q, rows, pixels_per_item, C, PC);
+    else
+        quantize_groups<1, LP><<<grid, block, 0, stream>>>(x, ths, q, rows, pixels_per_item, C, PC);
+}
+
+// The general-path kernel with the smallest group of lanes whose 4 channels a lane cover the widest word.
+void launch_quantize_groups(const float *x, const float *ths, int bitwidth, long rows, long pixels_per_item, int C, int PC,
+                            uint32_t *q, hipStream_t stream)
+{
+    const int widest = C < kWordBits ? C : kWordBits;
+    if (widest <= 4) launch_quantize_groups_of<1>(x, ths, bitwidth, rows, pixels_per_item, C, PC, q, stream);
+    else if (widest <= 8) launch_quantize_groups_of<2>(x, ths, bitwidth, rows, pixels_per_item, C, PC, q, stream);
+    else if (widest <= 16) launch_quantize_groups_of<4>(x, ths, bitwidth, rows, pixels_per_item, C, PC, q, stream);
+    else if (widest <= 32) launch_quantize_groups_of<8>(x, ths, bitwidth, rows, pixels_per_item, C, PC, q, stream);
+    else launch_quantize_groups_of<16>(x, ths, bitwidth, rows, pixels_per_item, C, PC, q, stream);
+}
+
 // x: fp32 [items][pixels_per_item][C]; qx: [items*pixels_per_item][PC][bitwidth];
 // btn: [items] or nullptr (then no counts are produced).
 hipError_t launch_quantize(const float *x, const float *ths, int bitwidth, long pixels_per_item,
@@ -502,6 +618,8 @@ hipError_t launch_quantize(const float *x, const float *ths, int bitwidth, long 
             else
                 quantize_rows64<1><<<grid, block, 0, stream>>>(x4, ths, q32, rows, words_per_item);
         }
+    } else if (pixels * PC < 0x7fffffffL) {
+        launch_quantize_groups(x, ths, bitwidth, pixels * PC, pixels_per_item, C, PC, reinterpret_cast<uint32_t *>(qx), stream);
     } else {
         const long units = pixels * PC;
         long blocks = (units + kWavesPerBlock - 1) / kWavesPerBlock;

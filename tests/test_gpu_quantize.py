@@ -26,6 +26,9 @@ def _run(x, ths, bitwidth, N, H, W, C):
     (64, 3, 3, 256),            # the notebook's weight tensor
     (1, 1, 1, 64), (7, 1, 3, 192),
     (2, 4, 5, 1), (2, 3, 3, 63), (3, 2, 2, 65), (2, 5, 3, 70), (1, 3, 3, 200),  # C % 64 != 0
+    # every lane-group width of the general path, full and ragged, several items per wave and waves per item
+    (3, 9, 11, 2), (2, 17, 13, 3), (5, 8, 8, 4), (2, 9, 7, 5), (3, 6, 5, 8), (2, 7, 9, 13), (4, 5, 5, 16),
+    (2, 6, 7, 17), (3, 5, 4, 31), (2, 8, 5, 32), (3, 4, 5, 33), (2, 13, 11, 100), (70, 2, 2, 129), (1, 40, 40, 3),
 ])
 def test_quantize_matches_oracle(bitwidth, shape):
     N, H, W, C = shape
