@@ -29,6 +29,7 @@ def _run(x, ths, bitwidth, N, H, W, C):
     # every lane-group width of the general path, full and ragged, several items per wave and waves per item
     (3, 9, 11, 2), (2, 17, 13, 3), (5, 8, 8, 4), (2, 9, 7, 5), (3, 6, 5, 8), (2, 7, 9, 13), (4, 5, 5, 16),
     (2, 6, 7, 17), (3, 5, 4, 31), (2, 8, 5, 32), (3, 4, 5, 33), (2, 13, 11, 100), (70, 2, 2, 129), (1, 40, 40, 3),
+    (5, 60, 61, 3), (3, 30, 31, 100), (4, 33, 35, 24),  # many workgroups, items ending inside a wave
 ])
 def test_quantize_matches_oracle(bitwidth, shape):
     N, H, W, C = shape
