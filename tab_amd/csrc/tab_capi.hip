@@ -215,6 +215,9 @@ static int conv_packed(const int64_t *dev_QX, const int64_t *dev_QW, const int32
     a.num = KH * KW * C;
     a.div_pc = tab::make_fastdiv((uint32_t)s.PC);
     a.div_kw = tab::make_fastdiv((uint32_t)KW);
+    a.div_pixels = tab::make_div32((uint32_t)(s.OH * s.OW));
+    a.div_ow = tab::make_div32((uint32_t)s.OW);
+    a.div_tiles_m = tab::make_div32(1);
     hipError_t e = tab::launch_conv(type, a, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return device_fail(e, "conv launch");
     return TAB_OK;

@@ -27,6 +27,27 @@ __device__ __forceinline__ uint32_t fastdiv(uint32_t x, FastDiv f)
     return f.d == 1 ? x : __umulhi(x, f.magic);
 }
 
+// Exact x / d for 0 <= x < 2^31 and 1 <= d < 2^31 with one 32x32 -> 64-bit multiply and a shift (a runtime
+// divisor otherwise costs some 25 instructions a lane): with s = ceil(log2 d) and mul = floor(2^(31+s) / d) + 1,
+// mul * d exceeds 2^(31+s) by at most d <= 2^s, so the quotient's error term x * (mul * d - 2^(31+s)) / (d * 2^(31+s))
+// stays below 1 / d for every x < 2^31.
+struct Div32 {
+    uint32_t mul, shift;
+};
+inline Div32 make_div32(uint32_t d)
+{
+    uint32_t s = 0;
+    while (((uint64_t)1 << s) < d) s++;
+    Div32 f;
+    f.shift = 31 + s;
+    f.mul = (uint32_t)((((uint64_t)1 << (31 + s)) / d) + 1);
+    return f;
+}
+__device__ __forceinline__ uint32_t div32(uint32_t x, Div32 f)
+{
+    return (uint32_t)(((uint64_t)x * f.mul) >> f.shift);
+}
+
 // Arguments of the fused pad + im2row + popcount-GEMM kernel.
 struct ConvArgs {
     const uint64_t *qx;  // packed activation [N][H][W][PC][APL]; PC = words per pixel and plane
@@ -48,6 +69,8 @@ struct ConvArgs {
     int num;       // KH*KW*C (BNN constant)
     int tiles_m;   // ceil(M / BM)
     FastDiv div_pc, div_kw;
+    Div32 div_pixels, div_ow;  // by OH*OW and OW: an output row's image and line
+    Div32 div_tiles_m;         // by tiles_m (set by the launchers with it)
 };
 
 // Launchers (tab_conv.hip / tab_quantize.hip); they enqueue on `stream` and return the

@@ -94,7 +94,7 @@ __global__ __launch_bounds__(kThreads) void conv_popcount(const ConvArgs p)
     const int tid = threadIdx.x;
     const int tx = tid & 15, ty = tid >> 4;
     // consecutive workgroups walk M first so neighbours share the weight tile in L2
-    const int tile_m = blockIdx.x % p.tiles_m, tile_n = blockIdx.x / p.tiles_m;
+    const int tile_n = (int)div32(blockIdx.x, p.div_tiles_m), tile_m = (int)blockIdx.x - tile_n * p.tiles_m;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
     Stager st;
@@ -279,6 +279,7 @@ hipError_t launch_tile(ConvArgs a, hipStream_t stream)
     a.kcw = (a.G + a.nchunks - 1) / a.nchunks;
     a.nchunks = (a.G + a.kcw - 1) / a.kcw;
     a.tiles_m = (a.M + BM - 1) / BM;
+    a.div_tiles_m = make_div32((uint32_t)a.tiles_m);
     const long tiles_n = (a.KN + BN - 1) / BN;
     const long blocks = (long)a.tiles_m * tiles_n;
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;

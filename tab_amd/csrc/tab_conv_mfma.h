@@ -146,7 +146,7 @@ __device__ __forceinline__ void conv_mfma_epilogue(const ConvArgs &p, f32x16 (&a
     for (int mt = 0; mt < TM; mt++) {
         th_row[mt] = 0.f;
         if (p.qy != nullptr) {
-            int n = (wave_m0 + mt * 32 + r) / (p.OH * p.OW);
+            int n = (int)div32((uint32_t)(wave_m0 + mt * 32 + r), p.div_pixels);
             n = n < p.N ? n : p.N - 1;  // rows past M are computed but not stored
             th_row[mt] = p.out_ths[n];
         }
@@ -299,7 +299,7 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
     const int kb = lane >> 5;  // which 32-bit half of the word this lane feeds
     const int ks = wave / (WM * WN);  // which words of every chunk this wave takes
     const int wm = (wave % (WM * WN)) % WM, wn = (wave % (WM * WN)) / WM;
-    const int tile_m = blockIdx.x % p.tiles_m, tile_n = blockIdx.x / p.tiles_m;
+    const int tile_n = (int)div32(blockIdx.x, p.div_tiles_m), tile_m = (int)blockIdx.x - tile_n * p.tiles_m;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
     Stager st;
@@ -403,6 +403,7 @@ hipError_t launch_mfma_tile(ConvArgs a, hipStream_t stream)
     a.kcw = KCH;
     a.nchunks = (a.G + KCH - 1) / KCH;
     a.tiles_m = (a.M + BM - 1) / BM;
+    a.div_tiles_m = make_div32((uint32_t)a.tiles_m);
     const long blocks = (long)a.tiles_m * ((a.KN + BN - 1) / BN);
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
     conv_mfma<TYPE, WM, WN, TM, TN, KCH, INTAP, KS><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);

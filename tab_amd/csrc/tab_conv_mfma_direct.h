@@ -65,12 +65,12 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int r = lane & 31, kb = lane >> 5;
     const int wm = wave % WM, wn = wave / WM;
-    const int tile_m = blockIdx.x % p.tiles_m, tile_n = blockIdx.x / p.tiles_m;
+    const int tile_n = (int)div32(blockIdx.x, p.div_tiles_m), tile_m = (int)blockIdx.x - tile_n * p.tiles_m;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
     // ---- what this lane fetches: granule idx = tid + i * 256 = (run * ROWS + row) * RUN + column ------
     const int pixels = p.OH * p.OW;
-    const int n_first = m0 / pixels;  // uniform
+    const int n_first = (int)div32((uint32_t)m0, p.div_pixels);  // uniform
     const size_t image_words = (size_t)p.H * p.W * p.PC * APL;
     const size_t a_bytes = (size_t)(p.N - n_first) * image_words * 8;
     const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
@@ -86,9 +86,9 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
         const int a_m = m0 + row;
         const bool live = granule < PA && a_m < p.M;
         const int mm = live ? a_m : m0;
-        const int n = mm / pixels;
+        const int n = (int)div32((uint32_t)mm, p.div_pixels);
         const int rem = mm - n * pixels;
-        const int oh = rem / p.OW, ow = rem - oh * p.OW;
+        const int oh = (int)div32((uint32_t)rem, p.div_ow), ow = rem - oh * p.OW;
         ih0[i] = live ? oh * p.s1 - p.p1 : -(1 << 30);  // a dead granule fails every bounds check
         iw0[i] = ow * p.s2 - p.p2;
         a_base[i] = (uint32_t)((((n - n_first) * p.H + (oh * p.s1 - p.p1)) * p.W + iw0[i]) * p.PC) * (uint32_t)(APL * 8) +
@@ -241,6 +241,7 @@ hipError_t launch_mfma_direct(ConvArgs a, hipStream_t stream)
     a.kcw = KCH;
     a.nchunks = a.G / KCH;
     a.tiles_m = (a.M + BM - 1) / BM;
+    a.div_tiles_m = make_div32((uint32_t)a.tiles_m);
     const long blocks = (long)a.tiles_m * ((a.KN + BN - 1) / BN);
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
     conv_mfma_direct<TYPE, WM, WN, TM, TN, KCH><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);

@@ -91,7 +91,7 @@ struct TileStager {
         // a wave shares its word index when the tile has at least 64 rows: the tap decode stays scalar
         a_w0 = BM >= 64 ? __builtin_amdgcn_readfirstlane(tid / BM) : tid / BM;
         const int pixels = p.OH * p.OW;
-        const int n_first = m0 / pixels;  // uniform
+        const int n_first = (int)div32((uint32_t)m0, p.div_pixels);  // uniform
         const size_t image_words = (size_t)p.H * p.W * p.PC * APL;
         const size_t a_bytes = (size_t)(p.N - n_first) * image_words * 8;
         a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(p.qx + (size_t)n_first * image_words), 0,
@@ -99,9 +99,9 @@ struct TileStager {
         const int a_m = m0 + a_row;
         const bool a_live = a_m < p.M;
         const int mm = a_live ? a_m : m0;
-        const int n = mm / pixels;
+        const int n = (int)div32((uint32_t)mm, p.div_pixels);
         const int r = mm - n * pixels;
-        const int oh = r / p.OW, ow = r - oh * p.OW;
+        const int oh = (int)div32((uint32_t)r, p.div_ow), ow = r - oh * p.OW;
         ih0 = a_live ? oh * p.s1 - p.p1 : -(1 << 30);  // a dead row fails every bounds check
         iw0 = ow * p.s2 - p.p2;
         a_base = (uint32_t)((((n - n_first) * p.H + (oh * p.s1 - p.p1)) * p.W + iw0) * p.PC) * (uint32_t)(APL * 8);
@@ -191,7 +191,7 @@ struct TapStager {
     __device__ __forceinline__ void init(const ConvArgs &p, int tid, int m0, int n0)
     {
         const int pixels = p.OH * p.OW;
-        const int n_first = m0 / pixels;  // uniform
+        const int n_first = (int)div32((uint32_t)m0, p.div_pixels);  // uniform
         const size_t image_words = (size_t)p.H * p.W * p.PC * APL;
         const size_t a_bytes = (size_t)(p.N - n_first) * image_words * 8;
         a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(p.qx + (size_t)n_first * image_words), 0,
@@ -203,9 +203,9 @@ struct TapStager {
             const int a_m = m0 + row;
             const bool live = row < BM && a_m < p.M;
             const int mm = live ? a_m : m0;
-            const int n = mm / pixels;
+            const int n = (int)div32((uint32_t)mm, p.div_pixels);
             const int r = mm - n * pixels;
-            const int oh = r / p.OW, ow = r - oh * p.OW;
+            const int oh = (int)div32((uint32_t)r, p.div_ow), ow = r - oh * p.OW;
             ih0[i] = live ? oh * p.s1 - p.p1 : -(1 << 30);  // a dead row fails every bounds check
             iw0[i] = ow * p.s2 - p.p2;
             a_base[i] = (uint32_t)((((n - n_first) * p.H + (oh * p.s1 - p.p1)) * p.W + iw0[i]) * p.PC) * (uint32_t)(APL * 8) +
