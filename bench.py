@@ -40,7 +40,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes moved by the ten conv launches of one headline step, from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE passes over `bench.py --profile` scaled by a 256 MiB copy
 # (profiles/quantize_conv_profile_sequence_traffic.txt).
-CONV_STEP_TRAFFIC_BYTES = 59368188
+CONV_STEP_TRAFFIC_BYTES = 59281150
 
 
 def valu_peak_tops(type):
