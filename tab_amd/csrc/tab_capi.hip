@@ -86,6 +86,9 @@ const char *tab_version(void) { return "tab_amd 0.1 gfx950"; }
 /* Tuning hook for benchmarking scripts; deliberately absent from include/tab_amd.h. */
 void tab_internal_force_conv_tile(int tm, int ng) { tab::force_conv_tile(tm, ng); }
 
+/* Test hook, likewise: the kernels' multiply-shift division evaluated on the host (x < 2^31, 1 <= d < 2^31). */
+uint32_t tab_internal_div32(uint32_t x, uint32_t d) { return tab::div32(x, tab::make_div32(d)); }
+
 int tab_set_conv_kernel(int kernel, int tile)
 {
     static const int popcount_tm[4] = {7, 8, 4, 2};  // 7: the popcount kernel's own choice

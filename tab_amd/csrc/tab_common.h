@@ -43,7 +43,7 @@ inline Div32 make_div32(uint32_t d)
     f.mul = (uint32_t)((((uint64_t)1 << (31 + s)) / d) + 1);
     return f;
 }
-__device__ __forceinline__ uint32_t div32(uint32_t x, Div32 f)
+__host__ __device__ __forceinline__ uint32_t div32(uint32_t x, Div32 f)
 {
     return (uint32_t)(((uint64_t)x * f.mul) >> f.shift);
 }

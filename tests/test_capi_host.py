@@ -143,3 +143,24 @@ def test_extension_module_names_and_cpu_rejection():
     assert "Conv2d" in public and "Quantize" in public
     with pytest.raises(RuntimeError, match="X must be a CUDA tensor"):
         TAB.Quantize(torch.zeros(1, 4, 4, 64), torch.zeros(1), 2, 1, 4, 4, 64)
+
+
+def test_multiply_shift_division_is_exact_below_2_31():
+    """The conv kernels decode output rows with x / d = (x * mul) >> shift; the same inline function evaluated on the
+    host must equal integer division for every divisor and numerator below 2^31, edge cases first."""
+    import random
+    lib = ctypes.CDLL(_capi.LIB_PATH)
+    f = lib.tab_internal_div32
+    f.argtypes = [ctypes.c_uint32, ctypes.c_uint32]
+    f.restype = ctypes.c_uint32
+    rng = random.Random(7)
+    top = 2 ** 31 - 1
+    divisors = list(range(1, 300)) + [2 ** k for k in range(31)] + [2 ** k + 1 for k in range(30)] + \
+        [2 ** k - 1 for k in range(2, 32)] + [784, 3136, 12544, 50176, 200704, 802816] + \
+        [rng.randrange(1, 2 ** 31) for _ in range(1500)]
+    for d in divisors:
+        xs = {0, 1, d - 1, d, min(d + 1, top), top, top - 1, (top // d) * d, max((top // d) * d - 1, 0)}
+        xs.update(rng.randrange(0, 2 ** 31) for _ in range(12))
+        xs.update(min(k * d + o, top) for k in (1, 2, 3, 7) for o in (-1, 0, 1) if k * d + o >= 0)
+        for x in xs:
+            assert f(x, d) == x // d, (x, d)
