@@ -68,7 +68,8 @@ int tab_out_extent(int in, int pad, int k, int stride);
  *   dev_X    fp32 [N*H*W*C]
  *   dev_ths  fp32 [>=N], threshold of item n is ths[n] (TAB_CPU.cpp:67,72)
  *   bitwidth 2: ternarize (v > t -> +1, else v < -t -> -1, else 0); 1: binarize (v < t -> -1)
- *   dev_QX   int64 [N*H*W*PC*bitwidth], every element is written
+ *   dev_QX   int64 [N*H*W*PC*bitwidth], aligned to a whole packed element (8*bitwidth bytes; the same holds
+ *            for tab_quantize_nchw, 16 bytes for tab_quantize_format); every element is written
  *   dev_BTN  int32 [N]; bitwidth 2: popcount of item n's nonzero plane (TAB_GEMM.cu:150-160,
  *            for every n); bitwidth 1: zeros (TAB_GEMM.cu:283)
  */

@@ -113,6 +113,8 @@ int tab_quantize(const float *dev_X, const float *dev_ths, int bitwidth, int N, 
     if (bitwidth != 1 && bitwidth != 2) return fail(TAB_ERR_BAD_ARGUMENT, "bitwidth must be 1 or 2, got %d", bitwidth);
     if (N < 1 || H < 1 || W < 1 || C < 1) return fail(TAB_ERR_BAD_ARGUMENT, "N, H, W, C must be positive");
     if (!dev_X || !dev_ths || !dev_QX || !dev_BTN) return fail(TAB_ERR_BAD_ARGUMENT, "null device pointer");
+    if (((uintptr_t)dev_X % 4) || ((uintptr_t)dev_QX % (8 * bitwidth)))
+        return fail(TAB_ERR_BAD_ARGUMENT, "X must be aligned to its floats and QX to a whole packed element (%d bytes)", 8 * bitwidth);
     hipError_t e = tab::launch_quantize(dev_X, dev_ths, bitwidth, (long)H * W, N, C,
                                         reinterpret_cast<uint64_t *>(dev_QX), dev_BTN,
                                         static_cast<hipStream_t>(stream));
@@ -126,6 +128,8 @@ int tab_quantize_nchw(const float *dev_X, const float *dev_ths, int bitwidth, in
     if (bitwidth != 1 && bitwidth != 2) return fail(TAB_ERR_BAD_ARGUMENT, "bitwidth must be 1 or 2, got %d", bitwidth);
     if (N < 1 || H < 1 || W < 1 || C < 1) return fail(TAB_ERR_BAD_ARGUMENT, "N, C, H, W must be positive");
     if (!dev_X || !dev_ths || !dev_QX || !dev_BTN) return fail(TAB_ERR_BAD_ARGUMENT, "null device pointer");
+    if (((uintptr_t)dev_X % 4) || ((uintptr_t)dev_QX % (8 * bitwidth)))
+        return fail(TAB_ERR_BAD_ARGUMENT, "X must be aligned to its floats and QX to a whole packed element (%d bytes)", 8 * bitwidth);
     if (((long)N * H * W + 255) / 256 * tab_packed_channels(C) > kMaxIndex)
         return fail(TAB_ERR_BAD_SHAPE, "tensor too large for one launch (N*H*W/256 * ceil(C/64) workgroups)");
     hipError_t e = tab::launch_quantize_nchw(dev_X, dev_ths, bitwidth, N, C, (long)H * W, reinterpret_cast<uint64_t *>(dev_QX),
@@ -174,6 +178,8 @@ int tab_quantize_format(const float *dev_X, const float *dev_ths, int type, int 
     if (type != TAB_DRF && type != TAB_RTN) return fail(TAB_ERR_BAD_ARGUMENT, "type must be 4 (DRF) or 5 (RTN), got %d", type);
     if (N < 1 || H < 1 || W < 1 || C < 1) return fail(TAB_ERR_BAD_ARGUMENT, "N, H, W, C must be positive");
     if (!dev_X || !dev_ths || !dev_QX) return fail(TAB_ERR_BAD_ARGUMENT, "null device pointer");
+    if (((uintptr_t)dev_X % 4) || ((uintptr_t)dev_QX % 16))
+        return fail(TAB_ERR_BAD_ARGUMENT, "X must be aligned to its floats and QX to 16 bytes");
     hipError_t e = tab::launch_quantize_format(dev_X, dev_ths, type, (long)H * W, N, C, reinterpret_cast<uint64_t *>(dev_QX),
                                                static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return device_fail(e, "quantize launch");

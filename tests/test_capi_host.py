@@ -58,6 +58,12 @@ def test_c_abi_rejects_bad_arguments_without_launching():
     assert b"bitwidth" in lib.tab_last_error()
     assert lib.tab_quantize(None, p, 2, 1, 1, 1, 64, p, p, None) == -1
     assert lib.tab_quantize(p, p, 2, 0, 1, 1, 64, p, p, None) == -1
+    # QX aligned to a whole packed element (8 bytes 1-bit, 16 bytes 2-bit and the type-4/5 formats)
+    assert lib.tab_quantize(p, p, 2, 1, 1, 1, 64, p + 8, p, None) == -1 and b"aligned" in lib.tab_last_error()
+    assert lib.tab_quantize(p, p, 1, 1, 1, 1, 64, p + 4, p, None) == -1
+    assert lib.tab_quantize(p + 2, p, 1, 1, 1, 1, 64, p, p, None) == -1
+    assert lib.tab_quantize_nchw(p, p, 2, 1, 64, 1, 1, p + 8, p, None) == -1
+    assert lib.tab_quantize_format(p, p, 4, 1, 1, 1, 64, p + 8, None) == -1 and b"aligned" in lib.tab_last_error()
     conv = lambda **kw: lib.tab_conv2d(  # noqa: E731
         kw.get("x", p), p, p, p, kw.get("type", 0), kw.get("p1", 1), 1, kw.get("s1", 1), 1,
         1, kw.get("H", 8), 8, 64, 4, 3, 3, p, kw.get("ws", p), kw.get("ws_bytes", 1 << 20), None)
