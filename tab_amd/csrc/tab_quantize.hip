@@ -112,7 +112,7 @@ template <int BITS, int LOADS = kLoadsPerLane>
 __global__ __launch_bounds__(kThreads) void quantize_rows64(const floatx4 *__restrict__ x,
                                                             const float *__restrict__ ths,
                                                             uint32_t *__restrict__ q, long rows,
-                                                            long rows_per_item)
+                                                            long rows_per_item, Div32 div_item)
 {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: so are row0 and the item test below
@@ -131,8 +131,11 @@ __global__ __launch_bounds__(kThreads) void quantize_rows64(const floatx4 *__res
         v[u] = __builtin_nontemporal_load(&x[(r < rows ? r : rows - 1) * 16 + l]);
     }
 
-    const long item_first = row0 / rows_per_item;
-    const bool one_item = (row_last / rows_per_item) == item_first;  // wave-uniform
+    // The wave's items (scalar; div_item.mul == 0 says that rows reach 2^31 and the division takes 64 bits): with the
+    // short division the threshold is in flight together with the loads of x instead of behind a long one.
+    const long item_first = div_item.mul ? (long)div32((uint32_t)row0, div_item) : row0 / rows_per_item;
+    const long item_last = div_item.mul ? (long)div32((uint32_t)row_last, div_item) : row_last / rows_per_item;
+    const bool one_item = item_last == item_first;
     const float t_first = ths[item_first];
 
     auto finish = [&](int u, float t) {
@@ -599,6 +602,7 @@ hipError_t launch_quantize(const float *x, const float *ths, int bitwidth, long 
     const bool fast = (C % kWordBits == 0) && ((uintptr_t)x % 16 == 0);
     if (fast) {
         const long rows = pixels * PC;
+        const Div32 div_item = rows < 0x7fffffffL ? make_div32((uint32_t)words_per_item) : Div32{0, 0};
         const long blocks = (rows + kRowsPerWave * kWavesPerBlock - 1) / (kRowsPerWave * kWavesPerBlock);
         const dim3 block(kThreads);
         const floatx4 *x4 = reinterpret_cast<const floatx4 *>(x);
@@ -608,15 +612,15 @@ hipError_t launch_quantize(const float *x, const float *ths, int bitwidth, long 
             // (3.1 MB of fp32: 5.5 -> 4.2 us)
             const dim3 grid((unsigned)((rows + 8 * kWavesPerBlock - 1) / (8 * kWavesPerBlock)));
             if (bitwidth == 2)
-                quantize_rows64<2, 2><<<grid, block, 0, stream>>>(x4, ths, q32, rows, words_per_item);
+                quantize_rows64<2, 2><<<grid, block, 0, stream>>>(x4, ths, q32, rows, words_per_item, div_item);
             else
-                quantize_rows64<1, 2><<<grid, block, 0, stream>>>(x4, ths, q32, rows, words_per_item);
+                quantize_rows64<1, 2><<<grid, block, 0, stream>>>(x4, ths, q32, rows, words_per_item, div_item);
         } else {
             const dim3 grid((unsigned)blocks);
             if (bitwidth == 2)
-                quantize_rows64<2><<<grid, block, 0, stream>>>(x4, ths, q32, rows, words_per_item);
+                quantize_rows64<2><<<grid, block, 0, stream>>>(x4, ths, q32, rows, words_per_item, div_item);
             else
-                quantize_rows64<1><<<grid, block, 0, stream>>>(x4, ths, q32, rows, words_per_item);
+                quantize_rows64<1><<<grid, block, 0, stream>>>(x4, ths, q32, rows, words_per_item, div_item);
         }
     } else if (pixels * PC < 0x7fffffffL) {
         launch_quantize_groups(x, ths, bitwidth, pixels * PC, pixels_per_item, C, PC, reinterpret_cast<uint32_t *>(qx), stream);
@@ -683,10 +687,11 @@ hipError_t launch_quantize_format(const float *x, const float *ths, int format, 
         const floatx4 *x4 = reinterpret_cast<const floatx4 *>(x);
         uint32_t *q32 = reinterpret_cast<uint32_t *>(qx);
         const long rows_per_item = pixels_per_item * (C / kWordBits);
+        const Div32 div_item = rows < 0x7fffffffL ? make_div32((uint32_t)rows_per_item) : Div32{0, 0};
         if (format == 4)
-            quantize_rows64<4><<<grid, block, 0, stream>>>(x4, ths, q32, rows, rows_per_item);
+            quantize_rows64<4><<<grid, block, 0, stream>>>(x4, ths, q32, rows, rows_per_item, div_item);
         else
-            quantize_rows64<5><<<grid, block, 0, stream>>>(x4, ths, q32, rows, rows_per_item);
+            quantize_rows64<5><<<grid, block, 0, stream>>>(x4, ths, q32, rows, rows_per_item, div_item);
         return hipGetLastError();
     }
     const long units = pixels * PC;
