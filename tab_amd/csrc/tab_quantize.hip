@@ -410,7 +410,7 @@ __global__ __launch_bounds__(kThreads) void quantize_nchw(const float *__restric
         for (int u = 0; u < kInFlight; u++) {
             const int j = j0 + u < channels ? j0 + u : channels - 1;  // clamped: the bit is masked below
             if (VEC == 1) {
-                v[u][0] = __builtin_nontemporal_load(src + (long)j * HW);
+                v[u][0] = src[(long)j * HW];  // the one-pixel form serves small tensors, likely cache-resident: plain loads
             } else {
                 const vec_t w = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(src + (long)j * HW));
 #pragma unroll
@@ -691,10 +691,17 @@ hipError_t launch_quantize_format(const float *x, const float *ths, int format, 
         uint32_t *q32 = reinterpret_cast<uint32_t *>(qx);
         const long rows_per_item = pixels_per_item * (C / kWordBits);
         const Div32 div_item = rows < 0x7fffffffL ? make_div32((uint32_t)rows_per_item) : Div32{0, 0};
-        if (format == 4)
+        if (blocks <= kSmallLaunchBlocks) {  // too small to fill the chip: 32 rows per workgroup, as in launch_quantize
+            const dim3 small((unsigned)((rows + 8 * kWavesPerBlock - 1) / (8 * kWavesPerBlock)));
+            if (format == 4)
+                quantize_rows64<4, 2><<<small, block, 0, stream>>>(x4, ths, q32, rows, rows_per_item, div_item);
+            else
+                quantize_rows64<5, 2><<<small, block, 0, stream>>>(x4, ths, q32, rows, rows_per_item, div_item);
+        } else if (format == 4) {
             quantize_rows64<4><<<grid, block, 0, stream>>>(x4, ths, q32, rows, rows_per_item, div_item);
-        else
+        } else {
             quantize_rows64<5><<<grid, block, 0, stream>>>(x4, ths, q32, rows, rows_per_item, div_item);
+        }
         return hipGetLastError();
     }
     const long units = pixels * PC;
