@@ -282,10 +282,7 @@ __global__ __launch_bounds__(kThreads) void quantize_groups(const float *__restr
         const uint32_t s_lo = or_reduce_group<LP>(w[0]), s_hi = LP == 16 ? or_reduce_group<LP>(w[1]) : 0u;
         if (BITS == 2) {
             const uint32_t n_lo = or_reduce_group<LP>(w[2]), n_hi = LP == 16 ? or_reduce_group<LP>(w[3]) : 0u;
-            if (r < rows && l == 0) {  // QX is aligned to its 8-byte words only
-                *reinterpret_cast<uintx2 *>(q + r * 4) = uintx2{s_lo, s_hi};
-                *reinterpret_cast<uintx2 *>(q + r * 4 + 2) = uintx2{n_lo, n_hi};
-            }
+            if (r < rows && l == 0) *reinterpret_cast<uintx4 *>(q + r * 4) = uintx4{s_lo, s_hi, n_lo, n_hi};
         } else {
             if (r < rows && l == 0) *reinterpret_cast<uintx2 *>(q + r * 2) = uintx2{s_lo, s_hi};
         }
