@@ -227,6 +227,7 @@ static int conv_packed(const int64_t *dev_QX, const int64_t *dev_QW, const int32
     a.div_pixels = tab::make_div32((uint32_t)(s.OH * s.OW));
     a.div_ow = tab::make_div32((uint32_t)s.OW);
     a.div_tiles_m = tab::make_div32(1);
+    a.tiles_n = 0;
     hipError_t e = tab::launch_conv(type, a, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return device_fail(e, "conv launch");
     return TAB_OK;

@@ -68,9 +68,10 @@ struct ConvArgs {
     int nchunks;   // ceil(G / kcw)
     int num;       // KH*KW*C (BNN constant)
     int tiles_m;   // ceil(M / BM)
+    int tiles_n;   // filter tiles when the workgroups are ordered by rows of Y (LDS-direct kernel, short K), else 0
+    Div32 div_tiles_m;  // by tiles_m, or by 8 * tiles_n in that order (set by the launchers)
     FastDiv div_pc, div_kw;
     Div32 div_pixels, div_ow;  // by OH*OW and OW: an output row's image and line
-    Div32 div_tiles_m;         // by tiles_m (set by the launchers with it)
 };
 
 // Launchers (tab_conv.hip / tab_quantize.hip); they enqueue on `stream` and return the
