@@ -271,6 +271,38 @@ __device__ __forceinline__ void conv_mfma_epilogue(const ConvArgs &p, f32x16 (&a
     }
 }
 
+// Workgroup -> tile.  Long K: the row tiles of one filter tile first, so that neighbours share the weight tile.
+// Short K and a large Y (p.tiles_n != 0; the launch is bound by writing Y): groups of eight row tiles walk the
+// filter tiles together, so that the workgroups running at one time write whole rows of Y rather than one
+// 512-byte column block of many rows (N=256 28x28x512->1024 1x1 BNN: 176 -> 150 us; N=32 56x56x256->1024: 110 -> 78).
+// False for the workgroups that pad the last group.
+__device__ __forceinline__ bool tile_of_workgroup(const ConvArgs &p, int &tile_m, int &tile_n)
+{
+    if (p.tiles_n != 0) {
+        const int group = (int)div32(blockIdx.x, p.div_tiles_m), in_group = (int)blockIdx.x - group * 8 * p.tiles_n;
+        tile_n = in_group >> 3;
+        tile_m = group * 8 + (in_group & 7);
+        return tile_m < p.tiles_m;
+    }
+    tile_n = (int)div32(blockIdx.x, p.div_tiles_m);
+    tile_m = (int)blockIdx.x - tile_n * p.tiles_m;
+    return true;
+}
+
+constexpr long kLargeY = 192L << 20;  // bytes of Y from which a short-K launch orders its workgroups by rows of Y
+
+// Chooses the order (a.tiles_m is set) and returns the number of workgroups.  From a sweep of 1x1 layers (C = 64..1024,
+// KN = 256..2048, N = 32..256): up to -30 % where Y is large and K a few words (a two-plane activation turns the gain
+// into a loss from 8 words on, a one-plane one from 16), +1-4 % where Y is a few tens of megabytes.
+template <int APL>
+long order_workgroups(ConvArgs &a, int tiles_n)
+{
+    const bool by_rows_of_y = tiles_n >= 2 && (long)a.M * a.KN * 4 >= kLargeY && a.G <= (APL == 1 ? 8 : 4);
+    a.tiles_n = by_rows_of_y ? tiles_n : 0;
+    a.div_tiles_m = make_div32((uint32_t)(by_rows_of_y ? 8 * tiles_n : a.tiles_m));
+    return by_rows_of_y ? (long)((a.tiles_m + 7) / 8) * 8 * tiles_n : (long)a.tiles_m * tiles_n;
+}
+
 // waves_per_eu: the shapes with four MFMA tiles per wave are capped at 128 registers, i.e. four
 // workgroups per CU (the 128x128 shape otherwise takes 136-152, 64 of them accumulators, and runs
 // three, measured 3-7 % slower); 256-row tiles need the state of more staged rows and get 168
@@ -299,7 +331,8 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
     const int kb = lane >> 5;  // which 32-bit half of the word this lane feeds
     const int ks = wave / (WM * WN);  // which words of every chunk this wave takes
     const int wm = (wave % (WM * WN)) % WM, wn = (wave % (WM * WN)) / WM;
-    const int tile_n = (int)div32(blockIdx.x, p.div_tiles_m), tile_m = (int)blockIdx.x - tile_n * p.tiles_m;
+    int tile_m, tile_n;
+    if (!tile_of_workgroup(p, tile_m, tile_n)) return;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
     Stager st;
@@ -403,8 +436,7 @@ hipError_t launch_mfma_tile(ConvArgs a, hipStream_t stream)
     a.kcw = KCH;
     a.nchunks = (a.G + KCH - 1) / KCH;
     a.tiles_m = (a.M + BM - 1) / BM;
-    a.div_tiles_m = make_div32((uint32_t)a.tiles_m);
-    const long blocks = (long)a.tiles_m * ((a.KN + BN - 1) / BN);
+    const long blocks = order_workgroups<Planes<TYPE>::A>(a, (a.KN + BN - 1) / BN);
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
     conv_mfma<TYPE, WM, WN, TM, TN, KCH, INTAP, KS><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
     return hipGetLastError();

@@ -65,20 +65,8 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int r = lane & 31, kb = lane >> 5;
     const int wm = wave % WM, wn = wave / WM;
-    // Workgroup -> tile.  Long K: the row tiles of one filter tile first, so that neighbours share the weight tile.
-    // Short K and a large Y (p.tiles_n != 0; the launch is bound by writing Y): groups of eight row tiles walk the filter tiles
-    // together, so that the workgroups running at one time write whole rows of Y rather than one 512-byte column
-    // block of many rows (N=256 28x28x512->1024 1x1: 176 -> 150 us).
     int tile_m, tile_n;
-    if (p.tiles_n != 0) {
-        const int group = (int)div32(blockIdx.x, p.div_tiles_m), in_group = (int)blockIdx.x - group * 8 * p.tiles_n;
-        tile_n = in_group >> 3;
-        tile_m = group * 8 + (in_group & 7);
-        if (tile_m >= p.tiles_m) return;
-    } else {
-        tile_n = (int)div32(blockIdx.x, p.div_tiles_m);
-        tile_m = (int)blockIdx.x - tile_n * p.tiles_m;
-    }
+    if (!tile_of_workgroup(p, tile_m, tile_n)) return;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
     // ---- what this lane fetches: granule idx = tid + i * 256 = (run * ROWS + row) * RUN + column ------
@@ -244,8 +232,6 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
     conv_mfma_epilogue<TYPE, TM, TN, KCH, 1>(p, acc, b_nonzero, wave_m0, wave_n0, lane, 0, nullptr);
 }
 
-constexpr long kLargeY = 192L << 20;  // bytes of Y from which a short-K launch orders its workgroups by rows of Y
-
 template <int TYPE, int WM, int WN, int TM, int TN, int KCH>
 hipError_t launch_mfma_direct(ConvArgs a, hipStream_t stream)
 {
@@ -256,14 +242,7 @@ hipError_t launch_mfma_direct(ConvArgs a, hipStream_t stream)
     a.kcw = KCH;
     a.nchunks = a.G / KCH;
     a.tiles_m = (a.M + BM - 1) / BM;
-    const int tiles_n = (a.KN + BN - 1) / BN;
-    // from a sweep of 1x1 layers (C = 64..1024, KN = 256..2048, N = 32..256): up to -30 % where Y is large and K a few
-    // words (a two-plane activation turns the gain into a loss from 8 words on, a one-plane one from 16), +1-4 %
-    // where Y is a few tens of megabytes
-    const bool by_rows_of_y = tiles_n >= 2 && (long)a.M * a.KN * 4 >= kLargeY && a.G <= (Planes<TYPE>::A == 1 ? 8 : 4);
-    a.tiles_n = by_rows_of_y ? tiles_n : 0;
-    a.div_tiles_m = make_div32((uint32_t)(by_rows_of_y ? 8 * tiles_n : a.tiles_m));
-    const long blocks = by_rows_of_y ? (long)((a.tiles_m + 7) / 8) * 8 * tiles_n : (long)a.tiles_m * tiles_n;
+    const long blocks = order_workgroups<Planes<TYPE>::A>(a, (a.KN + BN - 1) / BN);
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
     conv_mfma_direct<TYPE, WM, WN, TM, TN, KCH><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
     return hipGetLastError();
