@@ -196,6 +196,39 @@ def test_full_size_sweep_point_properties():
             assert bool(((y.to(torch.int64) - 9 * C) % 2 == 0).all())
 
 
+@pytest.mark.parametrize("C,KN", [(128, 384), (64, 256)])  # the LDS-direct kernel; the register-staged one (one word per pixel)
+def test_short_k_large_output_workgroup_order(C, KN):
+    """A 1x1 layer whose Y exceeds 192 MB orders its workgroups by rows of Y (groups of eight row tiles walk the
+    filter tiles), and 203840 = 65*56*56 rows leave the last group partly empty.  Too much for the oracle as a
+    whole: images are independent, so two images computed alone (the other order: their Y is small) must equal
+    the same images inside the batch, the first and the last image are compared with the oracle, and every
+    output obeys |y| <= C and, for BNN, y = C (mod 2)."""
+    N, H, W = 65, 56, 56
+    assert N * H * W * KN * 4 >= 192 << 20 and (N * H * W + 127) // 128 % 8 != 0
+    print(f"[case] short-K large-Y order N={N} {H}x{W}x{C}->{KN} 1x1, types 3 and 0", flush=True)
+    g = torch.Generator("cuda").manual_seed(3)
+    x = torch.randn((N, H, W, C), generator=g, device="cuda")
+    w = torch.randn((KN, 1, 1, C), generator=g, device="cuda")
+    for type in (3, 0):
+        ab, wb = act_bits(type), weight_bits(type)
+        x_ths = (0.7 * x.abs().reshape(N, -1).mean(dim=1)).contiguous() if ab == 2 else torch.zeros(N, device="cuda")
+        w_ths = (0.7 * w.abs().reshape(KN, -1).mean(dim=1)).contiguous() if wb == 2 else torch.zeros(KN, device="cuda")
+        QW, BTN = tab_amd.Quantize(w, w_ths, wb, KN, 1, 1, C)
+        y = tab_amd.Conv2d(x, QW, x_ths, BTN, type, 0, 0, 1, 1, N, H, W, C, KN, 1, 1)
+        for first in (0, N - 2):
+            part = tab_amd.Conv2d(x[first:first + 2].contiguous(), QW, x_ths[first:first + 2].contiguous(), BTN, type,
+                                  0, 0, 1, 1, 2, H, W, C, KN, 1, 1)
+            torch.cuda.synchronize()
+            assert torch.equal(y[first:first + 2], part)
+        for n in (0, N - 1):
+            want = oracle.conv2d(x[n:n + 1].cpu().numpy(), QW.cpu().numpy(), x_ths[n:n + 1].cpu().numpy(), BTN.cpu().numpy(),
+                                 type, 0, 0, 1, 1, 1, H, W, C, KN, 1, 1)
+            assert np.array_equal(y[n:n + 1].cpu().numpy(), want)
+        assert bool((y.abs() <= C).all())
+        if type == 3:
+            assert bool(((y.to(torch.int64) - C) % 2 == 0).all())
+
+
 def test_conv_rejects_wrong_sizes():
     x = torch.zeros((1, 4, 4, 64), device="cuda")
     ths = torch.zeros(1, device="cuda")
