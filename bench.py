@@ -41,7 +41,7 @@ HBM_PEAK_GBS = 8000.0
 # WRITE_SIZE passes over `bench.py --profile` scaled by a 256 MiB copy
 # (profiles/quantize_conv_profile_sequence_traffic.txt).
 STEPS_PER_GRAPH = 10  # steps captured into one HIP graph for the headline figure
-CONV_STEP_TRAFFIC_BYTES = 59281158
+CONV_STEP_TRAFFIC_BYTES = 59292389
 
 
 def valu_peak_tops(type):
