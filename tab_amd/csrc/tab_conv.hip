@@ -15,6 +15,8 @@
 // with the count accumulated in the instruction's addend.
 #include "tab_conv_stage.h"
 
+#include <atomic>
+
 namespace tab {
 namespace {
 
@@ -287,8 +289,15 @@ hipError_t launch_tile(ConvArgs a, hipStream_t stream)
     return hipGetLastError();
 }
 
-// Tuning hook (not part of the public ABI): forces one tile shape for every launch.
-int g_force_tm = 0, g_force_ng = 0;
+// Kernel choice of tab_set_conv_kernel, (tm << 8) | (ng + 1) in one atomic word so that a launch on another
+// thread sees either the old or the new pair, never a mix; 0 = the automatic choice.
+std::atomic<int> g_forced_kernel{0};
+struct Forced { int tm, ng; };
+inline Forced forced_kernel()
+{
+    const int v = g_forced_kernel.load(std::memory_order_relaxed);
+    return {v >> 8, (v & 0xff) - 1};
+}
 
 // Tile shapes.  Every shape keeps <= 128 VGPRs, i.e. at least 4 workgroups (4 waves per SIMD)
 // per CU; shapes with 128 accumulators at 2 waves per SIMD and 512-thread workgroups were
@@ -315,9 +324,10 @@ template <int TYPE>
 hipError_t launch_type(const ConvArgs &a, hipStream_t stream)
 {
     constexpr int BIG_BN = (TYPE == 0) ? 64 : 128;
-    if (g_force_tm == 8) return launch_big<TYPE>(a, stream);
-    if (g_force_tm == 4) return launch_tile<TYPE, 4, 1, 4, true>(a, stream);
-    if (g_force_tm == 2) return launch_tile<TYPE, 2, 1, 8, true>(a, stream);
+    const int force_tm = forced_kernel().tm;
+    if (force_tm == 8) return launch_big<TYPE>(a, stream);
+    if (force_tm == 4) return launch_tile<TYPE, 4, 1, 4, true>(a, stream);
+    if (force_tm == 2) return launch_tile<TYPE, 2, 1, 8, true>(a, stream);
     auto tiles = [&](int bm, int bn) { return (long)((a.M + bm - 1) / bm) * ((a.KN + bn - 1) / bn); };
     if (a.KN > BIG_BN / 2 && tiles(128, BIG_BN) >= 3072) return launch_big<TYPE>(a, stream);
     if (tiles(64, 64) >= 512) return launch_tile<TYPE, 4, 1, 4, true>(a, stream);
@@ -328,8 +338,7 @@ hipError_t launch_type(const ConvArgs &a, hipStream_t stream)
 
 void force_conv_tile(int tm, int ng)
 {
-    g_force_tm = tm;
-    g_force_ng = ng;
+    g_forced_kernel.store(tm == 0 ? 0 : ((tm << 8) | ((ng + 1) & 0xff)), std::memory_order_relaxed);
 }
 
 // fp32 accumulators hold integers up to 2^24 exactly; a product is at most 1 (9 for the 2-bit levels of
@@ -386,15 +395,17 @@ int conv_mfma_shape(int conv_type, const ConvArgs &a)
 
 hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream)
 {
+    const Forced forced = forced_kernel();
+    const int force_tm = forced.tm, force_ng = forced.ng;
     if (args.qy != nullptr) {  // packed output exists in the matrix-core kernel's 64-wide shapes only
         if (!conv_mfma_exact(args)) return hipErrorInvalidValue;
-        const int shape = (g_force_tm == 9 && g_force_ng >= 0 && g_force_ng != 3 && g_force_ng <= 6) ? g_force_ng : conv_mfma_shape(type, args);
+        const int shape = (force_tm == 9 && force_ng >= 0 && force_ng != 3 && force_ng <= 6) ? force_ng : conv_mfma_shape(type, args);
         return launch_conv_mfma(type, args, shape, stream);
     }
-    if (g_force_tm == 9) return launch_conv_mfma(type, args, g_force_ng < 0 ? conv_mfma_shape(type, args) : g_force_ng, stream);
+    if (force_tm == 9) return launch_conv_mfma(type, args, force_ng < 0 ? conv_mfma_shape(type, args) : force_ng, stream);
     // default path: matrix cores; the popcount kernel takes over when K is too long for exact fp32
     // accumulation (and when a benchmark forces one of its tiles)
-    if (g_force_tm == 0 && conv_mfma_exact(args)) return launch_conv_mfma(type, args, conv_mfma_shape(type, args), stream);
+    if (force_tm == 0 && conv_mfma_exact(args)) return launch_conv_mfma(type, args, conv_mfma_shape(type, args), stream);
     // types 4 and 5 exist on the matrix cores only
     if (type > 3) return launch_conv_mfma(type, args, conv_mfma_shape(type, args), stream);
     switch (type) {

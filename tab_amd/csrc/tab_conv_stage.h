@@ -136,8 +136,9 @@ struct TileStager {
         for (int i = 0; i < B_ITEMS; i++) {
             const int w = b_w0 + i * B_STEP;
             const int g = g0 + w;
-            const uint32_t word_off = (w < p.kcw && g < p.G) ? (uint32_t)g * (uint32_t)(BPL * 8) : kNoFilter;
-            b_reg[i] = load_item<BPL>(b_rsrc, b_base + word_off);
+            // select, not add: two out-of-range markers added together would wrap back into the range
+            const bool live = b_base != kNoFilter && w < p.kcw && g < p.G;
+            b_reg[i] = load_item<BPL>(b_rsrc, live ? b_base + (uint32_t)g * (uint32_t)(BPL * 8) : kNoFilter);
         }
     }
 
