@@ -129,7 +129,7 @@ size_t tab_conv2d_workspace_bytes(int type, int N, int H, int W, int C);
  *   dev_ths fp32 [>=N]
  *   dev_btn int32 [>=KN], read only for BTN (TAB_GEMM.cu:116); may be NULL otherwise
  *   dev_Y   fp32 [N*OH*OW*KN], OH = tab_out_extent(H, padding1, KH, stride1), OW likewise;
- *           every element is written
+ *           16-byte aligned (the kernels store four floats at a time); every element is written
  *   workspace / workspace_bytes: device scratch of at least tab_conv2d_workspace_bytes()
  *           bytes, 16-byte aligned; owned by the caller, reusable once the stream has
  *           passed this call
@@ -145,10 +145,33 @@ int tab_conv2d(const float *dev_X, const int64_t *dev_QW, const float *dev_ths,
                void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * tab_conv2d for callers that cannot allocate device memory or pass a workspace: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose
+ * ConvWithCuda_TAB cudaMallocs its scratch on every call, TAB_GEMM.cu:391-397).  Arguments and results are
+ * exactly tab_conv2d's; the packed activation goes to a scratch array built into the library
+ * (TAB_STATIC_SCRATCH_BYTES bytes of device memory per GPU, held until the process ends) instead of a
+ * caller-owned workspace.  The call allocates nothing and frees nothing.
+ *   - tab_conv2d_workspace_bytes(type, N, H, W, C) must not exceed TAB_STATIC_SCRATCH_BYTES, else
+ *     TAB_ERR_WORKSPACE and nothing is launched (use tab_conv2d with a workspace for larger activations).
+ *   - All calls on one GPU share that GPU's array: two calls whose kernels may overlap (different streams,
+ *     different host threads without ordering) race on it.  Calls on one stream are ordered and safe.
+ *   - The first call made on a device looks the array's address up once (no stream work, no allocation); make
+ *     that first call outside a graph capture.
+ */
+#define TAB_STATIC_SCRATCH_BYTES (32u << 20)
+size_t tab_static_scratch_bytes(void);
+int tab_conv2d_static(const float *dev_X, const int64_t *dev_QW, const float *dev_ths,
+                      const int32_t *dev_btn, int type, int padding1, int padding2, int stride1,
+                      int stride2, int N, int H, int W, int C, int KN, int KH, int KW, float *dev_Y,
+                      void *stream);
+
+/*
  * The second half of tab_conv2d on an activation that is already packed (the output of
  * tab_quantize with bitwidth 2 for TNN/TBN, 1 for BTN/BNN): zero padding, im2row and the
  * popcount GEMM (PadKernel + Img2RowKernel + GEMMWithCuda, TAB_GEMM.cuh:22-115) fused in
- * one kernel.  dev_QX int64 [N*H*W*PC*abits]; other arguments as in tab_conv2d.  Types 4 and 5:
+ * one kernel.  dev_QX int64 [N*H*W*PC*abits], aligned to a whole packed element (8*abits bytes; dev_QW likewise,
+ * 8*wbits bytes; dev_Y 16 bytes); other arguments as in tab_conv2d.  Unlike the reference's .toType() calls
+ * (TAB_GEMM.cu:341-347) no entry point converts element types: buffers must hold the types named here.  Types 4 and 5:
  * dev_QX int64 [N*H*W*tab_operand_words(type, 0, C)] from tab_quantize_format.
  */
 int tab_conv2d_packed(const int64_t *dev_QX, const int64_t *dev_QW, const int32_t *dev_btn,
@@ -163,7 +186,8 @@ int tab_conv2d_packed(const int64_t *dev_QX, const int64_t *dev_QW, const int32_
  * for bit, without Y ever reaching memory.  It chains layers packed-in / packed-out; the
  * reference has no counterpart (every TAB_Conv2d returns fp32 and the caller re-quantizes).
  *   dev_out_ths fp32 [>=N]: threshold for the outputs of image n
- *   dev_QY      int64 [N*OH*OW*ceil(KN/64)*out_bitwidth], every element is written
+ *   dev_QY      int64 [N*OH*OW*ceil(KN/64)*out_bitwidth], aligned to a whole packed element
+ *               (8*out_bitwidth bytes); every element is written
  * Types 0..3 only.
  */
 int tab_conv2d_packed_out(const int64_t *dev_QX, const int64_t *dev_QW, const int32_t *dev_btn,

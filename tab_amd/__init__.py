@@ -208,6 +208,43 @@ def Conv2d(X, QW, thresholds, btn, type, padding1, padding2, stride1, stride2, N
     return Y
 
 
+def static_scratch_bytes():
+    """Size of the scratch array built into the library that Conv2dStatic packs the activation into."""
+    return _lib.tab_static_scratch_bytes()
+
+
+def Conv2dStatic(X, QW, thresholds, btn, type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW, out=None):
+    """Conv2d through tab_conv2d_static: the packed activation goes to the library's built-in device scratch
+    (static_scratch_bytes() bytes per GPU) instead of a workspace tensor, so the C call allocates nothing.
+    With `out` (fp32, N*OH*OW*KN elements) given, this wrapper allocates nothing either.  Calls that may
+    overlap on one GPU race on the shared scratch."""
+    for t, name in ((X, "X"), (QW, "QW"), (thresholds, "thresholds"), (btn, "btn")):
+        _check_input(t, name)
+    _check_dtype(X, torch.float32, "X")
+    _check_dtype(QW, torch.int64, "QW")
+    _check_dtype(thresholds, torch.float32, "thresholds")
+    _check_dtype(btn, torch.int32, "btn")
+    (type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW) = (
+        int(v) for v in (type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW))
+    OH, OW = _conv_checks(QW, btn, type, N, H, W, C, KN, KH, KW, padding1, padding2, stride1, stride2)
+    if X.numel() != N * H * W * C:
+        raise RuntimeError(f"X has {X.numel()} elements, expected N*H*W*C = {N * H * W * C}")
+    if thresholds.numel() < N:
+        raise RuntimeError(f"thresholds has {thresholds.numel()} elements, expected at least N = {N}")
+    with torch.cuda.device(X.device):
+        if out is None:
+            out = torch.empty((N, KN, OH, OW), dtype=torch.float32, device=X.device)
+        else:
+            _check_input(out, "out")
+            _check_dtype(out, torch.float32, "out")
+            if out.numel() != N * KN * OH * OW:
+                raise RuntimeError(f"out has {out.numel()} elements, expected {N * KN * OH * OW}")
+        _capi.check(_lib, _lib.tab_conv2d_static(X.data_ptr(), QW.data_ptr(), thresholds.data_ptr(), btn.data_ptr(),
+                                                 type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW,
+                                                 out.data_ptr(), _stream()))
+    return out
+
+
 def Conv2dPacked(QX, QW, btn, type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW):
     """Conv2d on an activation already packed by Quantize (bitwidth 2 for types 0/1,
     1 for types 2/3) or by QuantizeFormat (types 4/5): the pad + im2row + GEMM stages of
@@ -276,6 +313,6 @@ def set_conv_kernel(kernel=CONV_AUTO, tile=-1):
 TAB_Quantize = Quantize
 TAB_Conv2d = Conv2d
 
-__all__ = ["Quantize", "QuantizeNCHW", "QuantizeFormat", "Conv2d", "Conv2dPacked", "Conv2dPackedOut", "Threshold", "TAB_Quantize", "TAB_Conv2d", "TabError",
+__all__ = ["Quantize", "QuantizeNCHW", "QuantizeFormat", "Conv2d", "Conv2dStatic", "static_scratch_bytes", "Conv2dPacked", "Conv2dPackedOut", "Threshold", "TAB_Quantize", "TAB_Conv2d", "TabError",
            "packed_channels", "out_shape", "version", "TNN", "TBN", "BTN", "BNN", "set_conv_kernel",
            "CONV_AUTO", "CONV_MATRIX", "CONV_POPCOUNT"]

@@ -5,6 +5,12 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <mutex>
+
+// Packed-activation scratch of tab_conv2d_static, one copy per GPU the library is loaded on.  In host code this
+// name is only a handle for hipGetSymbolAddress; the device address is looked up once per device (static_scratch
+// below) and that pointer is what the kernels get.
+static __device__ __align__(256) unsigned char scratch[TAB_STATIC_SCRATCH_BYTES];
 
 namespace {
 
@@ -83,10 +89,7 @@ const char *tab_last_error(void) { return g_last_error; }
 
 const char *tab_version(void) { return "tab_amd 0.1 gfx950"; }
 
-/* Tuning hook for benchmarking scripts; deliberately absent from include/tab_amd.h. */
-void tab_internal_force_conv_tile(int tm, int ng) { tab::force_conv_tile(tm, ng); }
-
-/* Test hook, likewise: the kernels' multiply-shift division evaluated on the host (x < 2^31, 1 <= d < 2^31). */
+/* Test hook, absent from include/tab_amd.h: the kernels' multiply-shift division evaluated on the host (x < 2^31, 1 <= d < 2^31). */
 uint32_t tab_internal_div32(uint32_t x, uint32_t d) { return tab::div32(x, tab::make_div32(d)); }
 
 int tab_set_conv_kernel(int kernel, int tile)
@@ -186,6 +189,17 @@ int tab_quantize_format(const float *dev_X, const float *dev_ths, int type, int 
     return TAB_OK;
 }
 
+/* Pointer checks shared by every conv entry point; they run before anything is launched. */
+static int check_conv_pointers(const ConvShape &s, int type, const void *dev_QX, const void *dev_QW, const void *dev_btn,
+                               const void *dev_Y, const void *dev_QY)
+{
+    if (!dev_QX || !dev_QW || (!dev_Y && !dev_QY)) return fail(TAB_ERR_BAD_ARGUMENT, "null device pointer");
+    if (type == TAB_BTN && !dev_btn) return fail(TAB_ERR_BAD_ARGUMENT, "btn is required for type 2 (BTN)");
+    if (((uintptr_t)dev_QX % (8 * s.abits)) || ((uintptr_t)dev_QW % (8 * s.wbits)) || ((uintptr_t)dev_Y % 16))
+        return fail(TAB_ERR_BAD_ARGUMENT, "QX/QW must be aligned to a whole packed element and Y to 16 bytes");
+    return TAB_OK;
+}
+
 /* Shared body of the packed-activation entry points: Y as fp32 (dev_Y) or thresholded and packed (dev_QY). */
 static int conv_packed(const int64_t *dev_QX, const int64_t *dev_QW, const int32_t *dev_btn, int type, int padding1,
                        int padding2, int stride1, int stride2, int N, int H, int W, int C, int KN, int KH, int KW,
@@ -194,10 +208,8 @@ static int conv_packed(const int64_t *dev_QX, const int64_t *dev_QW, const int32
     ConvShape s;
     int rc = check_conv(type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW, &s);
     if (rc != TAB_OK) return rc;
-    if (!dev_QX || !dev_QW || (!dev_Y && !dev_QY)) return fail(TAB_ERR_BAD_ARGUMENT, "null device pointer");
-    if (type == TAB_BTN && !dev_btn) return fail(TAB_ERR_BAD_ARGUMENT, "btn is required for type 2 (BTN)");
-    if (((uintptr_t)dev_QX % (8 * s.abits)) || ((uintptr_t)dev_QW % (8 * s.wbits)) || ((uintptr_t)dev_Y % 16))
-        return fail(TAB_ERR_BAD_ARGUMENT, "QX/QW must be aligned to a whole packed element and Y to 16 bytes");
+    rc = check_conv_pointers(s, type, dev_QX, dev_QW, dev_btn, dev_Y, dev_QY);
+    if (rc != TAB_OK) return rc;
     if (dev_QY) {
         if (type > 3) return fail(TAB_ERR_BAD_ARGUMENT, "packed output exists for types 0..3 only, got %d", type);
         if (out_bitwidth != 1 && out_bitwidth != 2)
@@ -252,21 +264,52 @@ int tab_conv2d_packed_out(const int64_t *dev_QX, const int64_t *dev_QW, const in
                        nullptr, dev_out_ths, out_bitwidth, dev_QY, stream);
 }
 
-int tab_conv2d(const float *dev_X, const int64_t *dev_QW, const float *dev_ths,
-               const int32_t *dev_btn, int type, int padding1, int padding2, int stride1,
-               int stride2, int N, int H, int W, int C, int KN, int KH, int KW, float *dev_Y,
-               void *workspace, size_t workspace_bytes, void *stream)
+/* Device address of `scratch` on the current device, looked up on the first call made with that device current. */
+static int static_scratch(void **out)
+{
+    constexpr int kMaxDevices = 64;
+    static std::mutex mutex;
+    static void *address[kMaxDevices] = {};
+    int device = -1;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) return device_fail(e, "hipGetDevice");
+    if (device < 0 || device >= kMaxDevices) return fail(TAB_ERR_DEVICE, "device index %d out of range", device);
+    std::lock_guard<std::mutex> lock(mutex);
+    if (address[device] == nullptr) {
+        void *ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return device_fail(e, "hipGetSymbolAddress(scratch)");
+        if (ptr == nullptr) return fail(TAB_ERR_DEVICE, "hipGetSymbolAddress(scratch) gave no address");
+        address[device] = ptr;
+    }
+    *out = address[device];
+    return TAB_OK;
+}
+
+/* Body of tab_conv2d and tab_conv2d_static (workspace == NULL and builtin: the library's own scratch): quantize
+ * into the workspace, then the fused conv kernel. */
+static int conv_from_floats(const float *dev_X, const int64_t *dev_QW, const float *dev_ths, const int32_t *dev_btn, int type,
+                            int padding1, int padding2, int stride1, int stride2, int N, int H, int W, int C, int KN, int KH,
+                            int KW, float *dev_Y, void *workspace, size_t workspace_bytes, bool builtin, void *stream)
 {
     ConvShape s;
     int rc = check_conv(type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW, &s);
     if (rc != TAB_OK) return rc;
     if (!dev_X || !dev_ths) return fail(TAB_ERR_BAD_ARGUMENT, "null device pointer");
+    if ((uintptr_t)dev_X % 4) return fail(TAB_ERR_BAD_ARGUMENT, "X must be aligned to its floats");
     const size_t need = tab_conv2d_workspace_bytes(type, N, H, W, C);
-    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace % 16))
+    if (builtin) {
+        if (need > TAB_STATIC_SCRATCH_BYTES)
+            return fail(TAB_ERR_WORKSPACE, "the packed activation needs %zu bytes, the built-in scratch holds %zu; use tab_conv2d with a workspace",
+                        need, (size_t)TAB_STATIC_SCRATCH_BYTES);
+        rc = static_scratch(&workspace);
+        if (rc != TAB_OK) return rc;
+    } else if (!workspace || workspace_bytes < need || ((uintptr_t)workspace % 16)) {
         return fail(TAB_ERR_WORKSPACE, "workspace must be 16-byte aligned and hold %zu bytes (got %zu)", need, workspace_bytes);
-    // A 1x1 convolution with stride and no padding reads one pixel in stride1*stride2: quantize only
-    // those, into a compact activation, and convolve it with stride 1 (same outputs, a fraction of
-    // the reads of X).
+    }
+    // everything the second stage would reject is rejected here, before the quantizer is enqueued
+    rc = check_conv_pointers(s, type, workspace, dev_QW, dev_btn, dev_Y, nullptr);
+    if (rc != TAB_OK) return rc;
     if (type > 3) {  // the CPU-only types: their own packers, then the same fused kernel
         hipError_t e = tab::launch_quantize_format(dev_X, dev_ths, type, (long)H * W, N, C, reinterpret_cast<uint64_t *>(workspace),
                                                    static_cast<hipStream_t>(stream));
@@ -274,6 +317,9 @@ int tab_conv2d(const float *dev_X, const int64_t *dev_QW, const float *dev_ths,
         return tab_conv2d_packed(reinterpret_cast<const int64_t *>(workspace), dev_QW, dev_btn, type, padding1, padding2, stride1,
                                  stride2, N, H, W, C, KN, KH, KW, dev_Y, stream);
     }
+    // A 1x1 convolution with stride and no padding reads one pixel in stride1*stride2: quantize only
+    // those, into a compact activation, and convolve it with stride 1 (same outputs, a fraction of
+    // the reads of X).
     if (KH == 1 && KW == 1 && padding1 == 0 && padding2 == 0 && (stride1 > 1 || stride2 > 1) && N * (long)s.OH < 65536 &&
         tab::quantize_strided_supported(dev_X, H, W, C, s.OH, s.OW)) {
         hipError_t e = tab::launch_quantize_strided(dev_X, dev_ths, s.abits, N, H, W, C, s.OH, s.OW, stride1, stride2,
@@ -291,6 +337,25 @@ int tab_conv2d(const float *dev_X, const int64_t *dev_QW, const float *dev_ths,
     return tab_conv2d_packed(reinterpret_cast<const int64_t *>(workspace), dev_QW, dev_btn, type,
                              padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW, dev_Y,
                              stream);
+}
+
+int tab_conv2d(const float *dev_X, const int64_t *dev_QW, const float *dev_ths,
+               const int32_t *dev_btn, int type, int padding1, int padding2, int stride1,
+               int stride2, int N, int H, int W, int C, int KN, int KH, int KW, float *dev_Y,
+               void *workspace, size_t workspace_bytes, void *stream)
+{
+    return conv_from_floats(dev_X, dev_QW, dev_ths, dev_btn, type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW,
+                            dev_Y, workspace, workspace_bytes, false, stream);
+}
+
+size_t tab_static_scratch_bytes(void) { return TAB_STATIC_SCRATCH_BYTES; }
+
+int tab_conv2d_static(const float *dev_X, const int64_t *dev_QW, const float *dev_ths, const int32_t *dev_btn, int type,
+                      int padding1, int padding2, int stride1, int stride2, int N, int H, int W, int C, int KN, int KH, int KW,
+                      float *dev_Y, void *stream)
+{
+    return conv_from_floats(dev_X, dev_QW, dev_ths, dev_btn, type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW,
+                            dev_Y, nullptr, 0, true, stream);
 }
 
 }  // extern "C"
