@@ -10,9 +10,13 @@ not built, the import fails.
 """
 try:
     from tab_amd._C import Conv2d, Quantize  # noqa: F401
+    # beyond the reference's two functions: the same C ABI, same conventions
+    from tab_amd._C import (Conv2dPacked, Conv2dPackedOut, QuantizeFormat, QuantizeNCHW,  # noqa: F401
+                            TAB_Conv2d, TAB_Quantize, Threshold)
 except ImportError as exc:  # pragma: no cover
     raise ImportError(
         "tab_amd/_C is not built; run `python -c 'import __graft_entry__ as g; g.build()'` first"
     ) from exc
 
-__all__ = ["Conv2d", "Quantize"]
+__all__ = ["Conv2d", "Quantize", "TAB_Conv2d", "TAB_Quantize", "QuantizeNCHW", "QuantizeFormat", "Threshold",
+           "Conv2dPacked", "Conv2dPackedOut"]

@@ -90,3 +90,63 @@ def test_extension_input_checks():
         TAB.Quantize(x, ths, 3, 1, 4, 4, 64)
     y = TAB.Conv2d(x, qw, ths, btn, 3, 1, 1, 1, 1, 1, 4, 4, 64, 4, 3, 3)
     assert tuple(y.shape) == (1, 4, 4, 4)
+
+
+def test_every_extension_entry_point_equals_ctypes_front_end():
+    """The pybind module exports everything the ctypes mirror does; each function, called through TAB_CUDA,
+    returns the tensors the mirror returns (same C ABI underneath), and Conv2d takes types 4 and 5 like the
+    reference's CPU binding (TAB_CPU.cpp:577-584, 621-633)."""
+    import TAB_CUDA as TAB
+
+    import tab_amd
+
+    assert {"QuantizeNCHW", "QuantizeFormat", "Threshold", "Conv2dPacked", "Conv2dPackedOut", "TAB_Quantize",
+            "TAB_Conv2d"} <= set(dir(TAB))
+    g = torch.Generator("cpu").manual_seed(11)
+    N, H, W, C, KN = 3, 10, 9, 192, 72
+    x = torch.randn([N, H, W, C], generator=g).cuda()
+    w = torch.randn([KN, 3, 3, C], generator=g).cuda()
+    # Threshold
+    ths_a, ths_b = TAB.Threshold(x, N, 0.7), tab_amd.Threshold(x, N, 0.7)
+    assert torch.equal(ths_a, ths_b) and torch.equal(TAB.Threshold(x, N), ths_b)
+    w_ths = TAB.Threshold(w, KN, 0.7)
+    # QuantizeNCHW
+    x_nchw = x.permute(0, 3, 1, 2).contiguous()
+    for bits in (1, 2):
+        qa, ba = TAB.QuantizeNCHW(x_nchw, ths_a, bits, N, C, H, W)
+        qb, bb = tab_amd.QuantizeNCHW(x_nchw, ths_a, bits, N, C, H, W)
+        qc, _ = TAB.Quantize(x, ths_a, bits, N, H, W, C)
+        assert torch.equal(qa, qb) and torch.equal(ba, bb) and torch.equal(qa, qc)
+    zeros = torch.zeros(max(N, KN), device="cuda")
+    for type in range(4):
+        print(f"[case] TAB_CUDA packed entry points type={type}", flush=True)
+        ab, wb = (2 if type < 2 else 1), (2 if type in (0, 2) else 1)
+        QW, BTN = TAB.Quantize(w, w_ths if wb == 2 else zeros, wb, KN, 3, 3, C)
+        QX, _ = TAB.Quantize(x, ths_a if ab == 2 else zeros, ab, N, H, W, C)
+        ya = TAB.Conv2dPacked(QX, QW, BTN, type, 1, 0, 1, 2, N, H, W, C, KN, 3, 3)
+        yb = tab_amd.Conv2dPacked(QX, QW, BTN, type, 1, 0, 1, 2, N, H, W, C, KN, 3, 3)
+        assert torch.equal(ya, yb) and tuple(ya.shape) == tuple(yb.shape)
+        assert torch.equal(ya, TAB.TAB_Conv2d(x, QW, ths_a if ab == 2 else zeros, BTN, type, 1, 0, 1, 2, N, H, W, C, KN, 3, 3))
+        out_ths = torch.full((N,), 3.0, device="cuda")
+        for out_bits in (1, 2):
+            qa = TAB.Conv2dPackedOut(QX, QW, BTN, type, 1, 0, 1, 2, N, H, W, C, KN, 3, 3, out_ths, out_bits)
+            qb = tab_amd.Conv2dPackedOut(QX, QW, BTN, type, 1, 0, 1, 2, N, H, W, C, KN, 3, 3, out_ths, out_bits)
+            assert torch.equal(qa, qb) and tuple(qa.shape) == tuple(qb.shape)
+    # types 4 and 5: packer and Conv2d
+    btn = torch.zeros(KN, dtype=torch.int32, device="cuda")
+    for type in (4, 5):
+        print(f"[case] TAB_CUDA types of the CPU path type={type}", flush=True)
+        xs, ws = (x.abs(), w.abs()) if type == 4 else (x, w)
+        x_t, w_t = torch.full((N,), 0.6, device="cuda"), torch.full((KN,), 0.5, device="cuda")
+        QWa, QWb = TAB.QuantizeFormat(ws, w_t, type, KN, 3, 3, C), tab_amd.QuantizeFormat(ws, w_t, type, KN, 3, 3, C)
+        assert torch.equal(QWa, QWb) and tuple(QWa.shape) == tuple(QWb.shape)
+        ya = TAB.Conv2d(xs, QWa, x_t, btn, type, 1, 1, 2, 1, N, H, W, C, KN, 3, 3)
+        yb = tab_amd.Conv2d(xs, QWa, x_t, btn, type, 1, 1, 2, 1, N, H, W, C, KN, 3, 3)
+        assert torch.equal(ya, yb)
+        qw_o = oracle.quantize_format(ws.cpu().numpy(), w_t.cpu().numpy(), type, KN, 3, 3, C)
+        want = oracle.conv2d(xs.cpu().numpy(), qw_o, x_t.cpu().numpy(), np.zeros(KN, np.int32), type, 1, 1, 2, 1, N, H, W, C, KN, 3, 3)
+        assert np.array_equal(ya.cpu().numpy(), want)
+        QX = TAB.QuantizeFormat(xs, x_t, type, N, H, W, C)
+        assert torch.equal(TAB.Conv2dPacked(QX, QWa, btn, type, 1, 1, 2, 1, N, H, W, C, KN, 3, 3), ya)
+    with pytest.raises(RuntimeError, match="types 0..3 only"):
+        TAB.Conv2dPackedOut(QX, QWa, btn, 4, 1, 1, 2, 1, N, H, W, C, KN, 3, 3, x_t, 1)
