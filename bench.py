@@ -37,11 +37,28 @@ ISSUED_CYCLES_PER_PAIR = {0: 12, 1: 6, 2: 6, 3: 6}
 # (TAB_GEMM.cu:48-51,81-84,113-114,142): TNN 5, TBN 4, BTN 3, BNN 2 lane-ops per pair.
 REFERENCE_MIX_OPS = {0: 5, 1: 4, 2: 3, 3: 2}
 HBM_PEAK_GBS = 8000.0
-# HBM bytes moved by the ten conv launches of one headline step, from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE passes over `bench.py --profile` scaled by a 256 MiB copy
-# (profiles/quantize_conv_profile_sequence_traffic.txt).
 STEPS_PER_GRAPH = 10  # steps captured into one HIP graph for the headline figure
-CONV_STEP_TRAFFIC_BYTES = 59292389
+HEADLINE_REPS = 7      # repetitions of the timed `steps` loop; the median is reported
+# HBM bytes moved by the ten conv launches of one headline step come from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes
+# over `bench.py --profile`, scaled by a 256 MiB copy; the summary of those passes is a tracked file that states the
+# figure on a line "conv_step_traffic_bytes = <n>".
+TRAFFIC_PROFILE = os.path.join("profiles", "quantize_conv_profile_sequence_traffic.txt")
+
+
+def profiled_step_traffic():
+    """(bytes, source) of the measured HBM traffic of one step's conv launches, read from the tracked profile summary;
+    (None, reason) when the file or the line is missing."""
+    import re
+
+    path = os.path.join(ROOT, TRAFFIC_PROFILE)
+    try:
+        for number, line in enumerate(open(path), 1):
+            m = re.match(r"\s*conv_step_traffic_bytes\s*=\s*(\d+)", line)
+            if m:
+                return int(m.group(1)), f"{TRAFFIC_PROFILE}:{number}"
+    except OSError:
+        return None, f"{TRAFFIC_PROFILE} not found"
+    return None, f"{TRAFFIC_PROFILE} has no conv_step_traffic_bytes line"
 
 
 def valu_peak_tops(type):
@@ -224,6 +241,90 @@ def cpu_baseline(oracle, layers, check_against=None, budget_s=10.0):
     return total_ops / total_s / 1e12, total_s, exact, passes
 
 
+def sampled_images(N, rows_per_image, min_rows=4096):
+    """Images whose output rows make up the correctness sample: at least `min_rows` rows (all of them when the batch
+    has fewer), always the first and the last image, the rest evenly spaced."""
+    k = min(N, max(2, -(-min_rows // rows_per_image)))
+    if k <= 1:
+        return [0]
+    return sorted({round(i * (N - 1) / (k - 1)) for i in range(k)})
+
+
+def gate(oracle, L, y=None):
+    """Bit-exact check of a layer's GPU output against the CPU oracle on sampled images (every output row of those
+    images, all KN filters, at least 4096 rows) and of the packed activation of the same images."""
+    import numpy as np
+
+    type, p1, p2, s1, s2, N, H, W, C, KN, KH, KW = L.args
+    if y is None:
+        y = L.conv2d()
+    OH, OW = out_extent(H, p1, KH, s1), out_extent(W, p2, KW, s2)
+    images = sampled_images(N, OH * OW)
+    qw, btn = L.QW.cpu().numpy(), L.BTN.cpu().numpy()
+    exact = True
+    for n in images:
+        x, ths = L.x[n:n + 1].cpu().numpy(), L.x_ths[n:n + 1].cpu().numpy()
+        want = oracle.conv2d(x, qw, ths, btn, type, p1, p2, s1, s2, 1, H, W, C, KN, KH, KW)
+        exact = exact and bool(np.array_equal(y[n:n + 1].cpu().numpy(), want))
+        qx, _ = oracle.quantize(x, ths, L.abits, 1, H, W, C)
+        exact = exact and bool(np.array_equal(L.QX[n:n + 1].cpu().numpy(), qx))
+    return {"bit_exact_vs_cpu": exact, "rows_checked": len(images) * OH * OW, "images_checked": len(images)}
+
+
+def cpu_reduced_batch(oracle, L, n_small=8):
+    """The CPU oracle on the first N' = min(N, 8) images of a layer, timed; the full-batch figure is the per-image time
+    times N (images are independent and equally expensive), labelled extrapolated when N' < N."""
+    type, p1, p2, s1, s2, N, H, W, C, KN, KH, KW = L.args
+    n = min(N, n_small)
+    x, ths = L.x[:n].cpu().numpy(), L.x_ths[:n].cpu().numpy()
+    qw, btn = L.QW.cpu().numpy(), L.BTN.cpu().numpy()
+    oracle.conv2d(x[:1], qw, ths[:1], btn, type, p1, p2, s1, s2, 1, H, W, C, KN, KH, KW)  # warm-up
+    best = None
+    for _ in range(2):
+        t0 = time.perf_counter()
+        oracle.conv2d(x, qw, ths, btn, type, p1, p2, s1, s2, n, H, W, C, KN, KH, KW)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    return {"cpu_ms": round(best / n * N * 1e3, 2), "cpu_tops": round(L.ops / N * n / best / 1e12, 3),
+            "cpu_images_timed": n, "extrapolated": n < N}
+
+
+def reference_gemm_baseline(oracle, L, budget_s=3.0):
+    """The reference's own BNNGEMM_baseline (TAB_CPU.cpp:312-328, compiled from the reference tree into
+    oracle/_ref/libtab_ref.so) on the im2row'd rows of one layer, beside this repository's port of the same GEMM on the
+    same rows and threads.  None when that library was not built."""
+    import numpy as np
+
+    if not oracle.have_ref():
+        return None
+    type, p1, p2, s1, s2, N, H, W, C, KN, KH, KW = L.args
+    assert type == 3
+    x, ths = L.host[0].numpy(), L.host[1].numpy()
+    qx, _ = oracle.quantize(x, ths, 1, N, H, W, C)
+    PC = (C + 63) // 64
+    rows = oracle.img2row(oracle.pad(qx, N, H, W, PC, p1, p2), N, H + 2 * p1, W + 2 * p2, PC, KH, KW, s1, s2)
+    M, K = rows.shape
+    qw = L.QW.cpu().numpy().reshape(KN, K)
+    ops = 2.0 * M * KN * K * 64
+    out = {}
+    for name, fn in (("reference", oracle.ref_gemm), ("port", oracle.gemm)):
+        y = fn(3, rows, qw, M, KN, K, NUM=KH * KW * C)  # warm-up, and the result to compare
+        out[name + "_y"] = y
+        spent, reps = 0.0, 0
+        while spent < budget_s / 2 and reps < 50:
+            t0 = time.perf_counter()
+            fn(3, rows, qw, M, KN, K, NUM=KH * KW * C)
+            spent += time.perf_counter() - t0
+            reps += 1
+        out[name] = ops * reps / spent / 1e12
+    return {"layer": layer_name(N, L.layer), "rows": int(M), "K_words": int(K),
+            "reference_BNNGEMM_baseline_tops": round(out["reference"], 4), "port_gemm_tops": round(out["port"], 4),
+            "threads": oracle.num_threads(), "results_equal": bool(np.array_equal(out["reference_y"], out["port_y"])),
+            "note": "GEMM stage only (rows already im2row'd), the reference's scalar popcount triple loop under its own "
+                    "'#pragma omp parallel for' against the port's; the reference's quantize and im2row are not timed "
+                    "(TAB_CPU.cpp as a whole does not compile)"}
+
+
 def profile_sequence(torch, tab):
     """Launch sequence for counter collection: a plain 256 MiB device copy (the yardstick that
     FETCH_SIZE / WRITE_SIZE are scaled with), Quantize at the roofline shape for both bit
@@ -259,6 +360,26 @@ def profile_sequence(torch, tab):
     print("profile sequence done")
 
 
+def timed_steps(torch, run_steps, steps, warmup_steps, reps=HEADLINE_REPS):
+    """Wall-clock seconds of `steps` steps, `reps` times over: run_steps(k) enqueues exactly k steps.  Warm-up: the
+    requested steps, then at least 20 ms of further steps (the first launches after an idle gap run at a lower
+    clock).  Each repetition is bracketed by a device synchronisation on both sides."""
+    run_steps(max(1, warmup_steps))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < 0.02:
+        run_steps(steps)
+        torch.cuda.synchronize()
+    times = []
+    for _ in range(reps):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        run_steps(steps)
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+    return times
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -290,49 +411,58 @@ def main():
         for l in layers:
             l.conv2d()
 
-    # eager: every call goes Python -> C ABI -> launch; host-bound for layers this small
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    eager_elapsed = time.perf_counter() - t0
+    def median_of(times):
+        return statistics.median(times)
 
-    # headline: the same step captured once into a HIP graph and replayed (the library only
-    # enqueues kernels on the current stream, so a caller can capture it)
+    # eager: every call goes Python -> C ABI -> launch; host-bound for layers this small
+    eager_times = timed_steps(torch, lambda k: [step() for _ in range(k)], args.steps, args.warmup, reps=3)
+    # ... and through the drop-in module a user of the reference imports (pybind11, tab_amd/_C)
+    import TAB_CUDA
+
+    def step_extension():
+        for l in layers:
+            TAB_CUDA.Conv2d(l.x, l.QW, l.x_ths, l.BTN, *l.args)
+
+    ext_times = timed_steps(torch, lambda k: [step_extension() for _ in range(k)], args.steps, args.warmup, reps=3)
+
+    # headline: the same step captured into a HIP graph and replayed (the library only enqueues kernels on the
+    # current stream, so a caller can capture it).  One step per graph ...
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         step()
-    for _ in range(args.warmup):
-        graph.replay()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        graph.replay()
-    torch.cuda.synchronize()
-    single_elapsed = time.perf_counter() - t0
+    single_times = timed_steps(torch, lambda k: [graph.replay() for _ in range(k)], args.steps, args.warmup)
     # ... and with STEPS_PER_GRAPH steps per graph, so that the graph launch (about 6 us a replay) is paid once per
-    # ten steps: the timed region is still exactly args.steps steps, every one of them recomputing all ten layers
+    # ten steps: a timed repetition is still exactly args.steps steps, every one of them recomputing all ten layers
     per_graph = min(STEPS_PER_GRAPH, args.steps)
     batch = torch.cuda.CUDAGraph()
     with torch.cuda.graph(batch):
         for _ in range(per_graph):
             step()
-    whole, rest = divmod(args.steps, per_graph)
-    for _ in range(max(1, args.warmup // per_graph)):
-        batch.replay()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(whole):
-        batch.replay()
-    for _ in range(rest):
-        graph.replay()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+
+    def replay_steps(k):
+        whole, rest = divmod(k, per_graph)
+        for _ in range(whole):
+            batch.replay()
+        for _ in range(rest):
+            graph.replay()
+
+    times = timed_steps(torch, replay_steps, args.steps, args.warmup)
+    elapsed = median_of(times)
     ms_per_step = elapsed / args.steps * 1e3
     value = total_ops * args.steps / elapsed / 1e12
+
+    # the same ten layers chained the way a binary network runs them: packed in, packed out, one launch per layer
+    packed_graph = torch.cuda.CUDAGraph()
+    for l in layers:
+        l.conv_packed_out()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(packed_graph):
+        for _ in range(per_graph):
+            for l in layers:
+                l.conv_packed_out()
+    packed_times = timed_steps(torch, lambda k: [packed_graph.replay() for _ in range(max(1, k // per_graph))],
+                               args.steps, args.warmup)
+    packed_steps = max(1, args.steps // per_graph) * per_graph
 
     # ---- per layer: latency of the whole call, kernel-only rates -------------------------
     per_layer, conv_ops, conv_ms = [], 0, 0.0
@@ -342,10 +472,12 @@ def main():
         q_ms = graph_time_ms(torch, l.quantize_only, 20)
         conv_ops += l.ops
         conv_ms += k_ms
+        kb = conv_kernel_bytes(N, l.layer)
         per_layer.append({"layer": layer_name(N, l.layer), "latency_us": round(call_ms * 1e3, 2),
                           "conv_kernel_us": round(k_ms * 1e3, 2), "quantize_kernel_us": round(q_ms * 1e3, 2),
                           "conv_kernel_tops": round(l.ops / k_ms / 1e9, 2),
                           "frac_mfma_peak": round(l.ops / k_ms / 1e9 / MFMA_FP4_PEAK_TOPS, 4),
+                          "conv_kernel_hbm_floor_us": round(kb / HBM_PEAK_GBS / 1e3, 2),
                           "hbm_floor_us": round(layer_bytes(N, l.layer) / HBM_PEAK_GBS / 1e3, 2)})
     achieved = conv_ops / conv_ms / 1e9  # TOP/s over the conv launches of one step
     # the same launches with the popcount kernel, for the comparison the matrix-core kernel has to win
@@ -360,14 +492,16 @@ def main():
     ridge = MFMA_FP4_PEAK_TOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
     achieved_gbs = conv_bytes / conv_ms / 1e6
     hbm_bound = intensity < ridge
+    traffic, traffic_source = profiled_step_traffic()
     roofline = {"kernel": "conv_mfma_direct<BNN> / conv_mfma<BNN> (v_mfma_f32_32x32x64_f8f6f4, FP4 operands)",
                 "bound": "hbm" if hbm_bound else "mfma",
                 "achieved": round(achieved_gbs if hbm_bound else achieved, 2),
                 "peak": HBM_PEAK_GBS if hbm_bound else MFMA_FP4_PEAK_TOPS,
                 "unit": "GB/s" if hbm_bound else "TFLOP/s",
                 "frac": round(achieved_gbs / HBM_PEAK_GBS if hbm_bound else achieved / MFMA_FP4_PEAK_TOPS, 4),
-                "traffic": CONV_STEP_TRAFFIC_BYTES,
+                "traffic": traffic, "traffic_source": traffic_source,
                 "algorithmic_bytes": conv_bytes,
+                "launches": len(layers), "sum_of_launch_durations_us": round(conv_ms * 1e3, 2),
                 "ops_per_byte": round(intensity, 1), "ridge_ops_per_byte": round(ridge, 1),
                 "mfma_achieved_tops": round(achieved, 2), "mfma_peak_tops": MFMA_FP4_PEAK_TOPS,
                 "mfma_frac": round(achieved / MFMA_FP4_PEAK_TOPS, 4),
@@ -381,9 +515,14 @@ def main():
                         "the same launches against the matrix-core peak.  At N=16 every launch is a few microseconds, "
                         "launch- and latency-bound (see resnet18_bnn_N256 and sweep_N256_28x28x512_3x3 for kernels long "
                         "enough to load the matrix cores, quantize for the HBM-bound kernel at its roofline shape); "
-                        "traffic = rocprofv3 FETCH_SIZE + WRITE_SIZE of the same ten launches, scaled by a copy; "
+                        "traffic = rocprofv3 FETCH_SIZE + WRITE_SIZE of the same ten launches, scaled by a copy, read from "
+                        "the tracked profile summary named in traffic_source (a separate profiler run, not this run); "
                         "popcount_kernel_achieved_tops is the VALU popcount kernel on the same launches, "
                         "valu_popcount_planning_peak its roofline (256 CU x 64 lanes x 2.4 GHz / 2 lane-ops per pair)"}
+
+    def rate(times_s, steps):
+        return {"tops": round(total_ops * steps / median_of(times_s) / 1e12, 3),
+                "ms_per_step": round(median_of(times_s) / steps * 1e3, 4)}
 
     result = {
         "metric": "tab_conv2d_effective_binary_tops", "value": round(value, 3), "unit": "TOP/s",
@@ -393,17 +532,69 @@ def main():
         "config": {"workload": "BNN (type 3) ResNet-18 layer set, N=16: 4x 3x3 s1 + 3x 3x3 s2 + 3x 1x1 s2; "
                                "one step = Conv2d (quantize + conv) on all 10 layers; ten steps per HIP graph replay",
                    "binary_ops_per_step": total_ops},
-        "eager": {"tops": round(total_ops * args.steps / eager_elapsed / 1e12, 3),
-                  "ms_per_step": round(eager_elapsed / args.steps * 1e3, 4),
-                  "note": "same step launched call by call from Python (host-bound)"},
-        "one_step_per_graph": {"tops": round(total_ops * args.steps / single_elapsed / 1e12, 3),
-                               "ms_per_step": round(single_elapsed / args.steps * 1e3, 4),
+        "timing": {"repetitions": len(times), "value_is": "median repetition of the timed steps loop",
+                   "ms_per_step_min": round(min(times) / args.steps * 1e3, 4),
+                   "ms_per_step_max": round(max(times) / args.steps * 1e3, 4),
+                   "warmup": f"{args.warmup} steps, then >= 20 ms of replays"},
+        "eager": {**rate(eager_times, args.steps), "note": "same step launched call by call from Python through the ctypes mirror (host-bound)"},
+        "eager_TAB_CUDA": {**rate(ext_times, args.steps),
+                           "note": "same step call by call through the drop-in pybind11 module TAB_CUDA.Conv2d (host-bound)"},
+        "one_step_per_graph": {**rate(single_times, args.steps),
                                "note": "the same steps with one graph replay per step: the graph launch adds about 6 us a step"},
+        "packed_in_packed_out_N16": {**rate(packed_times, packed_steps),
+                                     "note": "the same ten layers as Conv2dPackedOut (packed activation in, 1-bit packed output, "
+                                             "no quantize launch, no fp32 Y): 10 launches per step, ten steps per graph"},
         "roofline": roofline, "per_layer": per_layer,
     }
 
-    # ---- standalone Quantize at the HBM-roofline shape -------------------------------------
     if not args.quick:
+        import numpy as np
+
+        import oracle
+
+        # ---- correctness gate + CPU baseline of the headline workload: whole tensors, same tensors --------------
+        gpu_out = [l.conv2d().cpu().numpy() for l in layers]
+        tops, secs, exact, passes = cpu_baseline(oracle, layers, gpu_out)
+        result["cpu_baseline"] = {"value": round(tops, 4), "unit": "TOP/s", "cores": oracle.num_threads(),
+                                  "kind": "port",
+                                  "sample": f"the full workload (10 layers, N=16, {total_ops:.3e} binary ops per pass), "
+                                            f"{passes} passes in {secs:.2f} s: quantize + pad + im2row + popcount GEMM, "
+                                            "OpenMP over rows",
+                                  "gpu_bit_exact_vs_cpu": exact}
+        ref = reference_gemm_baseline(oracle, layers[1])
+        result["cpu_baseline"]["reference_gemm"] = ref if ref is not None else "oracle/_ref/libtab_ref.so not built: skipped"
+
+        # ---- the single-image TNN configuration: N=1, 32x32x64 -> 64, 3x3, pad 1 ------------------------------
+        L = Layer(tab, torch, 0, 1, (32, 32, 64, 64, 3, 3, 1, 1, 1, 1), seed=0)
+        call_ms = graph_time_ms(torch, L.conv2d, 20)
+        k_ms = graph_time_ms(torch, L.conv_kernel_only, 20)
+        result["tnn_single_image_32x32x64"] = {"latency_us": round(call_ms * 1e3, 2), "conv_kernel_us": round(k_ms * 1e3, 2),
+                                               "call_tops": round(L.ops / call_ms / 1e9, 2), **gate(oracle, L),
+                                               **cpu_reduced_batch(oracle, L)}
+
+        # ---- TBN and BTN on the ResNet-18 3x3 shapes, N=16, ReLU inputs (zero-heavy ternary planes) ------------
+        tern = {}
+        for type in (1, 2):
+            rows, t_ops, t_ms, t_cpu, ok = [], 0, 0.0, 0.0, True
+            for i, l in enumerate(RESNET18_LAYERS[:7]):
+                L = Layer(tab, torch, type, N, l, seed=40 + i, relu=True)
+                c_ms = graph_time_ms(torch, L.conv2d, 20)
+                k_ms = graph_time_ms(torch, L.conv_kernel_only, 20)
+                y = L.conv2d()
+                want = oracle.conv2d(L.host[0].numpy(), L.QW.cpu().numpy(), L.host[1].numpy(), L.BTN.cpu().numpy(), type, *L.args[1:])
+                ok = ok and bool(np.array_equal(y.cpu().numpy(), want))
+                cpu = cpu_reduced_batch(oracle, L, n_small=N)
+                t_ops += L.ops
+                t_ms += c_ms
+                t_cpu += cpu["cpu_ms"]
+                rows.append({"layer": layer_name(N, l), "latency_us": round(c_ms * 1e3, 2), "conv_kernel_us": round(k_ms * 1e3, 2),
+                             "conv_kernel_tops": round(L.ops / k_ms / 1e9, 1), "cpu_ms": cpu["cpu_ms"]})
+                del L
+            tern[TYPE_NAMES[type]] = {"call_tops": round(t_ops / t_ms / 1e9, 1), "cpu_tops": round(t_ops / t_cpu / 1e9, 3),
+                                      "bit_exact_vs_cpu": ok, "checked": "every output of every layer", "layers": rows}
+        result["resnet18_tbn_btn_relu_N16"] = tern
+
+        # ---- standalone Quantize at the HBM-roofline shape -------------------------------------
         qN, qH, qW, qC = 256, 56, 56, 256
         xq = torch.randn((qN, qH, qW, qC), generator=torch.Generator("cuda").manual_seed(0), device="cuda")
         quant = {}
@@ -411,14 +602,20 @@ def main():
             ths = (0.7 * xq.abs().reshape(qN, -1).mean(dim=1)).contiguous() if bitwidth == 2 else torch.zeros(qN, device="cuda")
             ms = event_time_ms(torch, lambda: tab.Quantize(xq, ths, bitwidth, qN, qH, qW, qC), 20)
             nbytes = 4 * qN * qH * qW * qC + 8 * qN * qH * qW * (qC // 64) * bitwidth + 8 * qN
+            qx, btn = tab.Quantize(xq, ths, bitwidth, qN, qH, qW, qC)
+            ok = True
+            for n in (0, qN // 2, qN - 1):  # whole images against the CPU quantizer
+                q_o, b_o = oracle.quantize(xq[n:n + 1].cpu().numpy(), ths[n:n + 1].cpu().numpy(), bitwidth, 1, qH, qW, qC)
+                ok = ok and bool(np.array_equal(qx[n:n + 1].cpu().numpy(), q_o)) and int(btn[n]) == int(b_o[0])
             quant[f"bitwidth{bitwidth}"] = {"us": round(ms * 1e3, 1), "GBps": round(nbytes / ms / 1e6, 1),
                                             "frac_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
-                                            "bytes": nbytes}
+                                            "bytes": nbytes, "bit_exact_vs_cpu": ok, "images_checked": 3}
             # the same values read as NCHW (256x256x56x56): the quantizer of PyTorch-layout callers
             xn = xq.view(qN, qC, qH, qW)
             ms = event_time_ms(torch, lambda: tab.QuantizeNCHW(xn, ths, bitwidth, qN, qC, qH, qW), 20)
             quant[f"nchw_bitwidth{bitwidth}"] = {"us": round(ms * 1e3, 1), "GBps": round(nbytes / ms / 1e6, 1),
                                                  "frac_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+            del qx
         ms = event_time_ms(torch, lambda: tab.Threshold(xq, qN, 0.7), 20)
         quant["threshold_abs_mean"] = {"us": round(ms * 1e3, 1), "GBps": round(4 * qN * qH * qW * qC / ms / 1e6, 1),
                                        "frac_hbm_peak": round(4 * qN * qH * qW * qC / ms / 1e6 / HBM_PEAK_GBS, 4)}
@@ -426,7 +623,7 @@ def main():
         result["quantize"] = {"shape": "256x56x56x256 fp32", "bound": "hbm", "peak_GBps": HBM_PEAK_GBS, **quant}
 
         # ---- the same ResNet-18 layer set at N=256 (kernels long enough not to be launch-bound)
-        rn_ops, rn_ms, rn_pop_ms, rn_out_ms, rn_call_ms, rn_layers = 0, 0.0, 0.0, 0.0, 0.0, []
+        rn_ops, rn_ms, rn_pop_ms, rn_out_ms, rn_call_ms, rn_layers, rn_ok, rn_cpu_ms = 0, 0.0, 0.0, 0.0, 0.0, [], True, 0.0
         for i, l in enumerate(RESNET18_LAYERS):
             L = Layer(tab, torch, 3, 256, l, seed=i, on_device=True)
             k_ms = graph_time_ms(torch, L.conv_kernel_only, 5, replays=4)
@@ -435,26 +632,36 @@ def main():
             p_ms = graph_time_ms(torch, L.conv_kernel_only, 5, replays=4)
             tab.set_conv_kernel(tab.CONV_AUTO, -1)
             o_ms = graph_time_ms(torch, L.conv_packed_out, 5, replays=4)
+            g = gate(oracle, L)
+            cpu = cpu_reduced_batch(oracle, L)
+            rn_ok = rn_ok and g["bit_exact_vs_cpu"]
+            rn_cpu_ms += cpu["cpu_ms"]
             rn_ops += L.ops
             rn_ms += k_ms
             rn_pop_ms += p_ms
             rn_out_ms += o_ms
             rn_call_ms += c_ms
             hbm_us = layer_bytes(256, l) / HBM_PEAK_GBS / 1e3
+            k_hbm_us = conv_kernel_bytes(256, l) / HBM_PEAK_GBS / 1e3
             rn_layers.append({"layer": layer_name(256, l), "conv_kernel_us": round(k_ms * 1e3, 1),
                               "call_us": round(c_ms * 1e3, 1), "conv_kernel_tops": round(L.ops / k_ms / 1e9, 1),
                               "popcount_kernel_tops": round(L.ops / p_ms / 1e9, 1),
                               "packed_out_us": round(o_ms * 1e3, 1), "packed_out_tops": round(L.ops / o_ms / 1e9, 1),
                               "frac_mfma_peak": round(L.ops / k_ms / 1e9 / MFMA_FP4_PEAK_TOPS, 4),
-                              "hbm_floor_us": round(hbm_us, 1), "call_frac_of_hbm_floor": round(hbm_us / (c_ms * 1e3), 4)})
+                              "conv_kernel_frac_of_hbm_peak": round(k_hbm_us / (k_ms * 1e3), 4),
+                              "hbm_floor_us": round(hbm_us, 1), "call_frac_of_hbm_floor": round(hbm_us / (c_ms * 1e3), 4),
+                              "rows_checked": g["rows_checked"], "cpu_ms_extrapolated": cpu["cpu_ms"]})
             del L
         result["resnet18_bnn_N256"] = {"conv_kernel_tops": round(rn_ops / rn_ms / 1e9, 1),
                                        "popcount_kernel_tops": round(rn_ops / rn_pop_ms / 1e9, 1),
                                        "call_tops": round(rn_ops / rn_call_ms / 1e9, 1),
                                        "packed_in_packed_out_tops": round(rn_ops / rn_out_ms / 1e9, 1),
+                                       "bit_exact_vs_cpu": rn_ok,
+                                       "cpu_tops_extrapolated_from_8_images": round(rn_ops / rn_cpu_ms / 1e9, 3),
                                        "note": "conv_kernel = Conv2dPacked (packed in, fp32 out); call = Conv2d (fp32 in, fp32 out: "
                                                "quantize + conv); packed_in_packed_out = Conv2dPackedOut (1-bit output packed in "
-                                               "the epilogue, what a chained binary layer runs)",
+                                               "the epilogue, what a chained binary layer runs); gate: every output row of "
+                                               "sampled images (>= 4096 rows per layer) and their packed activation against the CPU oracle",
                                        "frac_mfma_peak": round(rn_ops / rn_ms / 1e9 / MFMA_FP4_PEAK_TOPS, 4),
                                        "over_valu_planning_peak": round(rn_ops / rn_ms / 1e9 / planning_peak_tops(3), 4),
                                        "layers": rn_layers}
@@ -475,52 +682,56 @@ def main():
                                        "popcount_kernel_tops": round(L.ops / p_ms / 1e9, 1),
                                        "popcount_frac_valu_peak": round(L.ops / p_ms / 1e9 / valu_peak_tops(type), 4),
                                        "valu_planning_peak_tops": round(planning_peak_tops(type), 1),
-                                       "over_valu_planning_peak": round(L.ops / k_ms / 1e9 / planning_peak_tops(type), 4)}
+                                       "over_valu_planning_peak": round(L.ops / k_ms / 1e9 / planning_peak_tops(type), 4),
+                                       **gate(oracle, L), **cpu_reduced_batch(oracle, L)}
             del L
         result["sweep_N256_28x28x512_3x3"] = sweep
 
         # ---- more points of the large-batch sweep (the N = 64..256 benchmark configuration): conv kernel TOP/s ----
         # (C=KN, kernel, stride, pad1, pad2) at 28x28; asymmetric padding as the config asks
         points = [(256, 3, 1, 1, 0), (512, 3, 2, 1, 0), (512, 1, 1, 0, 0), (256, 1, 2, 1, 0)]
-        more = {}
-        for n_batch in (64, 256):
+        more, more_ok = {}, True
+        for n_batch in (64, 128, 256):
             for C, k, st, p1, p2 in points:
                 lay = (28, 28, C, C, k, k, p1, p2, st, st)
                 row = {}
                 for type in range(4):
                     L = Layer(tab, torch, type, n_batch, lay, seed=3, on_device=True)
                     row[TYPE_NAMES[type]] = round(L.ops / graph_time_ms(torch, L.conv_kernel_only, 5, replays=3) / 1e9, 1)
+                    more_ok = more_ok and gate(oracle, L)["bit_exact_vs_cpu"]
+                    if type == 3:
+                        row["cpu_BNN_tops_extrapolated"] = cpu_reduced_batch(oracle, L)["cpu_tops"]
                     del L
                 more[layer_name(n_batch, lay)] = row
+        more["bit_exact_vs_cpu"] = more_ok
         result["sweep_more_conv_kernel_tops"] = more
 
         # ---- TNN VGG-16-style stack at N=32 (the VGG benchmark configuration) ---------------------------
-        vgg, vgg_ops, vgg_ms, vgg_call_ms = [], 0, 0.0, 0.0
+        vgg, vgg_ops, vgg_ms, vgg_call_ms, vgg_ok, vgg_cpu_ms = [], 0, 0.0, 0.0, True, 0.0
         for i, (hw, c) in enumerate([(224, 64), (112, 128), (56, 256), (28, 512), (14, 512)]):
             lay = (hw, hw, c, c, 3, 3, 1, 1, 1, 1)
             L = Layer(tab, torch, 0, 32, lay, seed=20 + i, on_device=True)
             k_ms = graph_time_ms(torch, L.conv_kernel_only, 3, replays=3)
             c_ms = graph_time_ms(torch, L.conv2d, 3, replays=3)
+            g = gate(oracle, L)
+            cpu = cpu_reduced_batch(oracle, L, n_small=4)
+            vgg_ok = vgg_ok and g["bit_exact_vs_cpu"]
+            vgg_cpu_ms += cpu["cpu_ms"]
             vgg_ops += L.ops
             vgg_ms += k_ms
             vgg_call_ms += c_ms
             vgg.append({"layer": layer_name(32, lay), "conv_kernel_us": round(k_ms * 1e3, 1), "call_us": round(c_ms * 1e3, 1),
-                        "conv_kernel_tops": round(L.ops / k_ms / 1e9, 1)})
+                        "conv_kernel_tops": round(L.ops / k_ms / 1e9, 1), "rows_checked": g["rows_checked"],
+                        "cpu_ms_extrapolated": cpu["cpu_ms"]})
             del L
         result["vgg16_tnn_N32"] = {"conv_kernel_tops": round(vgg_ops / vgg_ms / 1e9, 1),
-                                   "call_tops": round(vgg_ops / vgg_call_ms / 1e9, 1), "layers": vgg}
-
-        # ---- CPU baseline: the oracle on the same layer set, same tensors --------------------
-        import oracle
-
-        gpu_out = [l.conv2d().cpu().numpy() for l in layers]
-        tops, secs, exact, passes = cpu_baseline(oracle, layers, gpu_out)
-        result["cpu_baseline"] = {"value": round(tops, 4), "unit": "TOP/s", "cores": oracle.num_threads(),
-                                  "kind": "port",
-                                  "sample": f"the full workload (10 layers, N=16, {total_ops:.3e} binary ops per pass), "
-                                            f"{passes} passes in {secs:.2f} s: quantize + pad + im2row + popcount GEMM, "
-                                            "OpenMP over rows",
-                                  "gpu_bit_exact_vs_cpu": exact}
+                                   "call_tops": round(vgg_ops / vgg_call_ms / 1e9, 1), "bit_exact_vs_cpu": vgg_ok,
+                                   "cpu_tops_extrapolated_from_4_images": round(vgg_ops / vgg_cpu_ms / 1e9, 3), "layers": vgg}
+        result["all_gates_bit_exact"] = bool(
+            result["cpu_baseline"]["gpu_bit_exact_vs_cpu"] and result["tnn_single_image_32x32x64"]["bit_exact_vs_cpu"]
+            and all(t["bit_exact_vs_cpu"] for t in tern.values()) and rn_ok and more_ok and vgg_ok
+            and all(v["bit_exact_vs_cpu"] for v in sweep.values())
+            and all(quant[f"bitwidth{b}"]["bit_exact_vs_cpu"] for b in (1, 2)))
     print(json.dumps(result))
 
 
