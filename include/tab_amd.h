@@ -202,7 +202,8 @@ int tab_conv2d_packed_out(const int64_t *dev_QX, const int64_t *dev_QW, const in
  *   TAB_CONV_AUTO      (tile -1) the library's choice: matrix cores, tile picked from the shape
  *   TAB_CONV_MATRIX    bit planes expanded to FP4 operands of v_mfma_f32_32x32x64_f8f6f4;
  *                      tile 0: 128x128, 1: 128x64, 2: 64x64, 3: 32x32 with K split over the
- *                      four waves, 4: 256x64, 5: 256x128, 6: 128x256; -1: picked from the shape
+ *                      four waves, 4: 256x64, 5: 256x128, 6: 128x256, 7: weights resident in registers
+ *                      (K of at most nine words; longer K takes the library's choice); -1: picked from the shape
  *   TAB_CONV_POPCOUNT  the reference's xor/and + popcount formulation on the vector ALU;
  *                      tile 0: big, 1: medium, 2: small; -1: picked from the shape
  *                      (types 4 and 5 exist on the matrix cores only and ignore this choice)

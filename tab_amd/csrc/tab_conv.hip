@@ -369,6 +369,11 @@ int conv_mfma_shape(int conv_type, const ConvArgs &a)
     // the CPU-only types follow the type with the same planes: 4 like TNN, 5 like BNN
     const int type = conv_type == 4 ? 0 : (conv_type == 5 ? 3 : conv_type);
     auto tiles = [&](int bm, int bn) { return (long)((a.M + bm - 1) / bm) * ((a.KN + bn - 1) / bn); };
+    // K of at most nine words and packed output: the kernel with the weights resident in registers, whose epilogue
+    // thresholds a pixel's filters inside a lane, runs 1.4-2x faster than the tiled shapes once the launch is a few
+    // rounds of waves (N=256 56x56x64->64 3x3: 24 against 38 us) and level with them on small ones; with fp32 output
+    // both are bound by writing Y and measure within 5 % of each other, so the tiled shapes keep those launches
+    if (conv_type <= 3 && a.G <= 9 && a.qy != nullptr && (a.M >= 65536 || a.G <= 2)) return 7;
     // short K: the per-tile prologue and epilogue weigh more, so a shape needs more tiles to pay
     const long enough = a.G >= 72 ? 192 : (a.G >= 36 ? 300 : 1024);
     // eight tiles per wave share each expanded operand between more MFMAs (the dearer operand gets the
@@ -399,7 +404,7 @@ hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream)
     const int force_tm = forced.tm, force_ng = forced.ng;
     if (args.qy != nullptr) {  // packed output exists in the matrix-core kernel's 64-wide shapes only
         if (!conv_mfma_exact(args)) return hipErrorInvalidValue;
-        const int shape = (force_tm == 9 && force_ng >= 0 && force_ng != 3 && force_ng <= 6) ? force_ng : conv_mfma_shape(type, args);
+        const int shape = (force_tm == 9 && force_ng >= 0 && force_ng != 3 && force_ng <= 7) ? force_ng : conv_mfma_shape(type, args);
         return launch_conv_mfma(type, args, shape, stream);
     }
     if (force_tm == 9) return launch_conv_mfma(type, args, force_ng < 0 ? conv_mfma_shape(type, args) : force_ng, stream);

@@ -488,12 +488,24 @@ hipError_t launch_mfma_shape(const ConvArgs &a, hipStream_t stream)
     }
 }
 
+// The short-K kernel with the weights resident in registers (tab_conv_mfma_regs.h), types 0..3.
+template <int TYPE>
+hipError_t launch_mfma_regs(const ConvArgs &a, hipStream_t stream);
+
 // shape: 0 = 128x128, 1 = 128x64, 2 = 64x64 (rows x filters per workgroup), 3 = 32x32 with the four
 // waves splitting every chunk of four words between them, 4 = 256x64, 5 = 256x128 and 6 = 128x256
-// (eight MFMA tiles per wave: fewer operand expansions per MFMA, half the occupancy)
+// (eight MFMA tiles per wave: fewer operand expansions per MFMA, half the occupancy), 7 = the register-resident
+// short-K kernel (K of at most nine words; longer K falls back to the shape picked from the launch)
 template <int TYPE>
 hipError_t launch_mfma_type(const ConvArgs &a, int shape, hipStream_t stream)
 {
+    if constexpr (TYPE <= 3) {
+        if (shape == 7) {
+            if (a.G <= 9) return launch_mfma_regs<TYPE>(a, stream);
+            shape = conv_mfma_shape(TYPE, a);
+            if (shape == 7) return hipErrorInvalidValue;
+        }
+    }
     switch (shape) {
     case 0: return launch_mfma_shape<TYPE, 2, 2, 2, 2>(a, stream);
     case 1: return launch_mfma_shape<TYPE, 4, 1, 1, 2>(a, stream);

@@ -250,3 +250,5 @@ hipError_t launch_mfma_direct(ConvArgs a, hipStream_t stream)
 
 }  // namespace
 }  // namespace tab
+
+#include "tab_conv_mfma_regs.h"

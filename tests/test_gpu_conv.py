@@ -95,7 +95,7 @@ def test_large_channel_layers(type, case):
     _conv_case(type, *case)
 
 
-KERNEL_VARIANTS = [(tab_amd.CONV_MATRIX, t) for t in range(7)] + [(tab_amd.CONV_POPCOUNT, t) for t in range(3)]
+KERNEL_VARIANTS = [(tab_amd.CONV_MATRIX, t) for t in range(8)] + [(tab_amd.CONV_POPCOUNT, t) for t in range(3)]
 VARIANT_CASES = [
     (2, 9, 6, 70, 5, 3, 3, 1, 0, 1, 2),        # one word per pixel pair: chunks cross taps
     (2, 12, 12, 192, 130, 3, 3, 1, 1, 1, 1),   # PC = 3: odd words per tap
@@ -120,6 +120,54 @@ def test_every_kernel_variant(type, variant, restore_kernel_choice):
     tab_amd.set_conv_kernel(*variant)
     for case in VARIANT_CASES:
         _conv_case(type, *case, seed=11 + type, relu=(type == 1))
+
+
+SHORT_K_CASES = [
+    # K of at most nine words: the kernel with the weights resident in registers, one wave per 32 output pixels
+    (2, 12, 12, 64, 64, 3, 3, 1, 1, 1, 1),     # 9 words, the C = 64 3x3 shape
+    (3, 9, 7, 33, 70, 3, 3, 1, 0, 2, 1),       # tail bits in the only word, ragged KN, tiles spanning images
+    (2, 10, 10, 128, 100, 2, 2, 1, 1, 1, 1),   # 8 words as 2x2 taps of two words
+    (1, 7, 9, 192, 33, 1, 3, 0, 1, 1, 1),      # 9 words as 1x3 taps of three words
+    (5, 3, 3, 64, 31, 3, 3, 1, 1, 1, 1),       # 45 output pixels over five images: two tiles, the second partly empty
+    (2, 8, 8, 320, 130, 1, 1, 0, 0, 1, 1),     # 5 words run as 8
+    (2, 8, 8, 192, 65, 1, 1, 1, 1, 1, 1),      # 3 words run as 4, padded 1x1
+    (4, 6, 6, 512, 256, 1, 1, 0, 0, 1, 1),     # 8 words, four filter tiles
+    (2, 9, 9, 64, 1, 3, 3, 2, 2, 3, 3),        # one filter, pad 2, stride 3
+    (1, 5, 5, 100, 7, 1, 1, 0, 0, 1, 1),       # 2 words
+    (3, 4, 4, 64, 64, 1, 1, 0, 0, 1, 1),       # 1 word
+]
+
+
+@pytest.mark.parametrize("type", [0, 1, 2, 3])
+@pytest.mark.parametrize("case", SHORT_K_CASES)
+def test_short_k_register_resident_kernel(type, case, restore_kernel_choice):
+    tab_amd.set_conv_kernel(tab_amd.CONV_MATRIX, 7)
+    _conv_case(type, *case, seed=21 + type, relu=(type == 1))
+
+
+@pytest.mark.parametrize("type", [0, 3])
+def test_short_k_waves_walk_several_tiles(type):
+    """100352 output pixels are 3136 tiles of 32, more than the waves of a launch: waves loop over tile, tile + waves.
+    Too slow for the oracle as a whole: images computed alone equal the same images in the batch; first and last image
+    against the oracle."""
+    N, H, W, C, KN = 32, 56, 56, 64, 64
+    g = torch.Generator("cuda").manual_seed(type)
+    x = torch.randn((N, H, W, C), generator=g, device="cuda")
+    w = torch.randn((KN, 3, 3, C), generator=g, device="cuda")
+    ab, wb = act_bits(type), weight_bits(type)
+    x_ths = (0.7 * x.abs().reshape(N, -1).mean(dim=1)).contiguous() if ab == 2 else torch.zeros(N, device="cuda")
+    w_ths = (0.7 * w.abs().reshape(KN, -1).mean(dim=1)).contiguous() if wb == 2 else torch.zeros(KN, device="cuda")
+    QW, BTN = tab_amd.Quantize(w, w_ths, wb, KN, 3, 3, C)
+    y = tab_amd.Conv2d(x, QW, x_ths, BTN, type, 1, 1, 1, 1, N, H, W, C, KN, 3, 3)
+    for first in (0, 15, N - 1):
+        part = tab_amd.Conv2d(x[first:first + 1].contiguous(), QW, x_ths[first:first + 1].contiguous(), BTN, type,
+                              1, 1, 1, 1, 1, H, W, C, KN, 3, 3)
+        torch.cuda.synchronize()
+        assert torch.equal(y[first:first + 1], part)
+    for n in (0, N - 1):
+        want = oracle.conv2d(x[n:n + 1].cpu().numpy(), QW.cpu().numpy(), x_ths[n:n + 1].cpu().numpy(), BTN.cpu().numpy(),
+                             type, 1, 1, 1, 1, 1, H, W, C, KN, 3, 3)
+        assert np.array_equal(y[n:n + 1].cpu().numpy(), want)
 
 
 def test_kernel_variants_agree_on_random_bits(restore_kernel_choice):

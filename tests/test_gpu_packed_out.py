@@ -65,7 +65,7 @@ def test_packed_out(type, case, out_bits):
         _packed_out_case(type, *case, out_bits, kind, seed=type + out_bits)
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 4, 5, 6])
+@pytest.mark.parametrize("tile", [0, 1, 2, 4, 5, 6, 7])
 @pytest.mark.parametrize("type", [0, 3])
 def test_packed_out_every_tile(type, tile, restore_kernel_choice):
     tab_amd.set_conv_kernel(tab_amd.CONV_MATRIX, tile)
@@ -113,3 +113,22 @@ def test_packed_out_rejects_bad_arguments():
         tab_amd.Conv2dPackedOut(QX, QW, btn, 3, 1, 1, 1, 1, N, H, W, C, KN, 3, 3, torch.zeros(0, device="cuda"), 1)
     with pytest.raises(RuntimeError, match="dtype"):
         tab_amd.Conv2dPackedOut(QX, QW, btn, 3, 1, 1, 1, 1, N, H, W, C, KN, 3, 3, ths.double(), 1)
+
+
+SHORT_K_PACKED = [
+    # K of at most nine words (the register-resident kernel's own packed epilogue)
+    (2, 12, 12, 64, 64, 3, 3, 1, 1, 1, 1),     # 9 words, one word of filters
+    (3, 9, 7, 33, 70, 3, 3, 1, 0, 2, 1),       # ragged KN: the second word holds six filters, tiles span images
+    (2, 8, 8, 320, 130, 1, 1, 0, 0, 1, 1),     # three words of filters, the last with two
+    (5, 3, 3, 64, 31, 3, 3, 1, 1, 1, 1),       # fewer than 32 filters
+    (4, 6, 6, 512, 256, 1, 1, 0, 0, 1, 1),     # four full words
+    (1, 5, 5, 100, 97, 1, 1, 0, 0, 1, 1),      # 97 filters: one half-word used in the last word
+]
+
+
+@pytest.mark.parametrize("out_bits", [1, 2])
+@pytest.mark.parametrize("type", [0, 1, 2, 3])
+@pytest.mark.parametrize("case", SHORT_K_PACKED)
+def test_packed_out_short_k(type, case, out_bits):
+    for kind in ("zero", "integer", "fraction"):
+        _packed_out_case(type, *case, out_bits, kind, seed=3 * type + out_bits)
