@@ -1,8 +1,9 @@
 // Matrix-core microbenchmark for the conv roofline: (1) checks that the FP4 (E2M1) encodings the conv
 // kernel builds from packed bit planes multiply to exact integers in v_mfma_f32_32x32x64_f8f6f4 for
 // all four operand combinations, (2) measures the instruction's issue rate alone and with the
-// per-tile expansion work of each conv type in front of it (2x2 tiles per wave, as in the kernel's
-// 128x128 shape).  Register-resident: no memory traffic in the timed loops.
+// per-tile expansion work of each conv type in front of it, for the tiles per wave and workgroups per CU the conv
+// kernel runs (2x2 at up to four workgroups, 4x2 / 2x4 at two), (3) measures how many independent vector
+// instructions fit in an MFMA's shadow.  Register-resident: no memory traffic in the timed loops.
 #include <hip/hip_runtime.h>
 #include <cstdio>
 #include <cstdint>
@@ -54,44 +55,82 @@ __global__ void k_check(const uint32_t *As, const uint32_t *Az, const uint32_t *
     for (int j = 0; j < 4; j++)
         for (int i = 0; i < 4; i++) C[(8 * j + 4 * kb + i) * 32 + r] = c[4 * j + i];
 }
-// MODE 0: mfma only; 1: BNN expansions; 2: TNN expansions; 3: TBN
-template <int MODE>
+// MODE 0: mfma only; 1: BNN expansions; 2: TNN expansions; 3: TBN.  TM x TN MFMA tiles per wave, one expansion per
+// operand tile and step as in the conv kernel: 2x2 (the 128x128 workgroup tile), 4x2 and 2x4 (256x128 / 128x256).
+template <int MODE, int TM, int TN>
 __global__ __launch_bounds__(256) void k_tput(float *out, int iters, uint32_t seed)
 {
-    v16f c[2][2];
-    for (int i = 0; i < 2; i++) for (int j = 0; j < 2; j++) for (int e = 0; e < 16; e++) c[i][j][e] = 0;
-    uint32_t w[8];
-    for (int i = 0; i < 8; i++) w[i] = seed * (threadIdx.x + 1) * (2 * i + 1);
-    v8i a[2], b[2];
-    for (int i = 0; i < 2; i++) { a[i] = bin_a(w[i]); b[i] = bin_b(w[2 + i]); }
+    v16f c[TM][TN];
+    for (int i = 0; i < TM; i++) for (int j = 0; j < TN; j++) for (int e = 0; e < 16; e++) c[i][j][e] = 0;
+    uint32_t w[2 * (TM + TN)];
+    for (int i = 0; i < 2 * (TM + TN); i++) w[i] = seed * (threadIdx.x + 1) * (2 * i + 1);
+    v8i a[TM], b[TN];
+    for (int i = 0; i < TM; i++) a[i] = bin_a(w[i]);
+    for (int i = 0; i < TN; i++) b[i] = bin_b(w[TM + i]);
     for (int it = 0; it < iters; it++) {
         if (MODE != 0) {
-            for (int i = 0; i < 2; i++) {
-                a[i] = (MODE == 1) ? bin_a(w[i]) : ter_a(w[i], w[4 + i]);
-                b[i] = (MODE == 2) ? ter_b(w[2 + i], w[6 + i]) : bin_b(w[2 + i]);
-            }
-            w[0] += 0x9e3779b9u; for (int i = 1; i < 8; i++) w[i] ^= w[i - 1];
+            for (int i = 0; i < TM; i++) a[i] = (MODE == 1) ? bin_a(w[i]) : ter_a(w[i], w[TM + TN + i]);
+            for (int i = 0; i < TN; i++) b[i] = (MODE == 2) ? ter_b(w[TM + i], w[2 * TM + TN + i]) : bin_b(w[TM + i]);
+            w[0] += 0x9e3779b9u; for (int i = 1; i < 2 * (TM + TN); i++) w[i] ^= w[i - 1];
         }
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+        for (int i = 0; i < TM; i++)
 #pragma unroll
-            for (int j = 0; j < 2; j++) c[i][j] = mfma(a[i], b[j], c[i][j]);
+            for (int j = 0; j < TN; j++) c[i][j] = mfma(a[i], b[j], c[i][j]);
     }
     float s = 0;
-    for (int i = 0; i < 2; i++) for (int j = 0; j < 2; j++) for (int e = 0; e < 16; e++) s += c[i][j][e];
+    for (int i = 0; i < TM; i++) for (int j = 0; j < TN; j++) for (int e = 0; e < 16; e++) s += c[i][j][e];
     if (s == 12345.678f) out[threadIdx.x] = s;
 }
-template <int MODE> int tput(const char *name, int bpc)
+template <int MODE, int TM, int TN> int tput(const char *name, int bpc)
 {
     float *out; CK(hipMalloc(&out, 4096));
     const int iters = 4000, blocks = 256 * bpc;
     hipEvent_t e0, e1; CK(hipEventCreate(&e0)); CK(hipEventCreate(&e1));
-    k_tput<MODE><<<blocks, 256>>>(out, 10, 3); CK(hipDeviceSynchronize());
-    CK(hipEventRecord(e0)); k_tput<MODE><<<blocks, 256>>>(out, iters, 3); CK(hipEventRecord(e1)); CK(hipEventSynchronize(e1));
+    k_tput<MODE, TM, TN><<<blocks, 256>>>(out, 10, 3); CK(hipDeviceSynchronize());
+    CK(hipEventRecord(e0)); k_tput<MODE, TM, TN><<<blocks, 256>>>(out, iters, 3); CK(hipEventRecord(e1)); CK(hipEventSynchronize(e1));
     float ms; CK(hipEventElapsedTime(&ms, e0, e1));
-    double macs = (double)blocks * 4 * iters * 4 * 32 * 32 * 64;
-    printf("%-28s blocks/CU=%d %.3f ms  %.0f binary-equivalent TOP/s; cycles per MFMA per SIMD @2.4GHz = %.1f\n", name, bpc, ms,
-           2 * macs / (ms * 1e-3) / 1e12, ms * 1e-3 * 2.4e9 / ((double)bpc * iters * 4));
+    double macs = (double)blocks * 4 * iters * TM * TN * 32 * 32 * 64;
+    printf("%-16s tiles/wave=%dx%d blocks/CU=%d %.3f ms  %.0f binary-equivalent TOP/s; cycles per MFMA per SIMD @2.4GHz = %.1f\n", name, TM, TN,
+           bpc, ms, 2 * macs / (ms * 1e-3) / 1e12, ms * 1e-3 * 2.4e9 / ((double)bpc * iters * TM * TN));
+    CK(hipFree(out));
+    return 0;
+}
+// What fits in an MFMA's shadow: eight independent MFMAs per round, each followed by NV pairs of vector instructions
+// (shift, and-or: the expansion's instructions) on registers the MFMAs do not read.
+template <int NV>
+__global__ __launch_bounds__(256) void k_shadow(float *out, int iters, uint32_t seed)
+{
+    v16f c[8];
+    for (int i = 0; i < 8; i++) for (int e = 0; e < 16; e++) c[i][e] = 0;
+    uint32_t w[8];
+    for (int i = 0; i < 8; i++) w[i] = seed * (threadIdx.x + 1) * (2 * i + 1);
+    const v8i a = {1, 2, 3, 4, 0, 0, 0, 0}, b = {5, 6, 7, 8, 0, 0, 0, 0};
+    uint32_t mask = M3, pat = M1;
+    asm volatile("" : "+s"(mask));
+    asm volatile("" : "+v"(pat));
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int m = 0; m < 8; m++) {
+            c[m] = mfma(a, b, c[m]);
+#pragma unroll
+            for (int v = 0; v < NV; v++) w[(m * NV + v) & 7] = ((w[(m * NV + v) & 7] << 1) & mask) | pat;
+        }
+    }
+    float s = 0;
+    for (int i = 0; i < 8; i++) { for (int e = 0; e < 16; e++) s += c[i][e]; s += (float)w[i]; }
+    if (s == 12345.678f) out[threadIdx.x] = s;
+}
+template <int NV> int shadow(int bpc)
+{
+    float *out; CK(hipMalloc(&out, 4096));
+    const int iters = 2000, blocks = 256 * bpc;
+    hipEvent_t e0, e1; CK(hipEventCreate(&e0)); CK(hipEventCreate(&e1));
+    k_shadow<NV><<<blocks, 256>>>(out, 10, 3); CK(hipDeviceSynchronize());
+    CK(hipEventRecord(e0)); k_shadow<NV><<<blocks, 256>>>(out, iters, 3); CK(hipEventRecord(e1)); CK(hipEventSynchronize(e1));
+    float ms; CK(hipEventElapsedTime(&ms, e0, e1));
+    printf("mfma + %2d independent vector instructions each, blocks/CU=%d: cycles per MFMA per SIMD @2.4GHz = %.1f\n", 2 * NV, bpc,
+           ms * 1e-3 * 2.4e9 / ((double)bpc * iters * 8));
     CK(hipFree(out));
     return 0;
 }
@@ -122,6 +161,13 @@ int main()
         }
         printf("check A %s x B %s: %d mismatches of 1024 (C[0][0]=%g)\n", (mode & 1) ? "ternary" : "binary", (mode & 2) ? "ternary" : "binary", bad, hC[0]);
     }
-    for (int bpc : {1, 2, 3}) { tput<0>("f4 mfma only", bpc); tput<1>("BNN expansions", bpc); tput<3>("TBN expansions", bpc); tput<2>("TNN expansions", bpc); }
+    // 2x2 tiles per wave run up to four workgroups per CU in the conv kernel, eight tiles per wave two
+    for (int bpc : {1, 2, 3, 4}) {
+        tput<0, 2, 2>("f4 mfma only", bpc); tput<1, 2, 2>("BNN expansions", bpc); tput<3, 2, 2>("TBN expansions", bpc); tput<2, 2, 2>("TNN expansions", bpc);
+    }
+    for (int bpc : {1, 2}) {
+        tput<1, 4, 2>("BNN expansions", bpc); tput<3, 2, 4>("TBN expansions", bpc); tput<2, 4, 2>("TNN expansions", bpc);
+    }
+    for (int bpc : {2, 4}) { shadow<0>(bpc); shadow<1>(bpc); shadow<2>(bpc); shadow<3>(bpc); shadow<4>(bpc); shadow<6>(bpc); }
     return 0;
 }
