@@ -328,7 +328,8 @@ def reference_gemm_baseline(oracle, L, budget_s=3.0):
 def profile_sequence(torch, tab):
     """Launch sequence for counter collection: a plain 256 MiB device copy (the yardstick that
     FETCH_SIZE / WRITE_SIZE are scaled with), Quantize at the roofline shape for both bit
-    widths, the conv kernel of every ResNet-18 N=16 layer, and the conv kernel of the large
+    widths, Conv2d (quantizer launch + conv launch) on every ResNet-18 N=16 layer, the short-K layer
+    N=256 56x56x64->64 with fp32 and with packed output, and the conv kernel of the large
     sweep point for all four types: the default (matrix-core) kernel, then the popcount kernel on
     the same tensors.  Three repetitions each."""
     src = torch.empty(256 * 1024 * 1024 // 4, dtype=torch.float32, device="cuda").normal_()
@@ -344,10 +345,18 @@ def profile_sequence(torch, tab):
         tab.Quantize(xq, zeros, 1, qN, qH, qW, qC)
         tab.Quantize(xq, ths, 2, qN, qH, qW, qC)
     del xq
-    for i, l in enumerate(RESNET18_LAYERS):
-        L = Layer(tab, torch, 3, 16, l, seed=i)
+    layers = [Layer(tab, torch, 3, 16, l, seed=i) for i, l in enumerate(RESNET18_LAYERS)]
+    torch.cuda.synchronize()
+    for L in layers:
         for _ in range(3):
-            L.conv_kernel_only()
+            L.conv2d()
+    del layers
+    L = Layer(tab, torch, 3, 256, RESNET18_LAYERS[0], seed=0, on_device=True)
+    for _ in range(3):
+        L.conv_kernel_only()
+    for _ in range(3):
+        L.conv_packed_out()
+    del L
     for type in range(4):
         L = Layer(tab, torch, type, 256, (28, 28, 512, 512, 3, 3, 1, 1, 1, 1), seed=7, on_device=True)
         for kernel in (tab.CONV_AUTO, tab.CONV_POPCOUNT):
