@@ -66,6 +66,9 @@ int check_conv(int type, int p1, int p2, int s1, int s2, int N, int H, int W, in
     const long image_bytes = (long)H * W * s->PC * s->abits * 8;
     if (image_bytes * (256 / ((long)s->OH * s->OW) + 2) > 0xffffffffL)
         return fail(TAB_ERR_BAD_SHAPE, "packed image of %ld bytes is too large for 32-bit offsets", image_bytes);
+    // a wave addresses its (at most 128) rows of Y with 32-bit byte offsets below 2 GiB
+    if ((long)KN * 4 * 128 >= (1L << 31))
+        return fail(TAB_ERR_BAD_SHAPE, "KN=%d is too large for 32-bit offsets into a tile of Y", KN);
     return TAB_OK;
 }
 

@@ -151,7 +151,6 @@ __device__ __forceinline__ void conv_mfma_epilogue(const ConvArgs &p, f32x16 (&a
             th_row[mt] = p.out_ths[n];
         }
     }
-    const bool whole = wave_m0 + 32 * TM <= p.M && wave_n0 + 32 * TN <= p.KN;  // wave-uniform
     if (KS > 1) {
         // the KS waves hold partial sums of the same tile: exchange them through LDS; wave ks
         // finishes rows 8*ks .. 8*ks+7
@@ -246,27 +245,34 @@ __device__ __forceinline__ void conv_mfma_epilogue(const ConvArgs &p, f32x16 (&a
         }
         return;
     }
+    // fp32 output through a buffer descriptor over the wave's rows of Y: rows past M lie past its end and
+    // columns past KN get an offset past it, so every store is unconditional (a branch per store, which
+    // "if (in range) store" compiles to, cost more than the store: the epilogue of a 256x128 tile took 6.5 us)
+    const long rows_left = (long)p.M - wave_m0;
+    if (rows_left <= 0) return;  // wave-uniform
+    const size_t y_bytes = (size_t)(rows_left < 32 * TM ? rows_left : 32 * TM) * p.KN * 4;  // < 2 GiB (launch check)
+    const __amdgpu_buffer_rsrc_t y_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(p.y + (size_t)wave_m0 * p.KN), 0, (int)y_bytes, kBufferFlags);
+    const uint32_t row_bytes = (uint32_t)p.KN * 4u;
 #pragma unroll
     for (int nt = 0; nt < TN; nt++) {
         const int col = wave_n0 + nt * 32 + r;
-        const bool col_ok = col < p.KN;
         float bias = 0.f;
         if (TYPE == 2) {
             const int nonzero = b_nonzero[nt] + __shfl_xor(b_nonzero[nt], 32, 64);
             bias = (float)(btn_col[nt] - nonzero);
         }
         if (TYPE == 3) bias = (float)(p.num - 64 * p.nchunks * KCH);
-        float *out = p.y + (size_t)(wave_m0 + 4 * kb) * p.KN + col;
+        // kNoFilter + any offset inside the tile stays out of range without wrapping
+        const uint32_t lane_off = col < p.KN ? (uint32_t)(4 * kb) * row_bytes + (uint32_t)col * 4u : kNoFilter;
 #pragma unroll
         for (int mt = 0; mt < TM; mt++)
 #pragma unroll
             for (int j = 0; j < 4; j++)
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    const int row = mt * 32 + 8 * j + i;  // + 4*kb, already in `out`
-                    const float v = acc[mt][nt][4 * j + i] + bias;
-                    if (whole) out[(size_t)row * p.KN] = v;
-                    else if (col_ok && wave_m0 + 4 * kb + row < p.M) out[(size_t)row * p.KN] = v;
+                    const int row = mt * 32 + 8 * j + i;  // + 4*kb, already in lane_off
+                    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[mt][nt][4 * j + i] + bias), y_rsrc,
+                                                          lane_off + (uint32_t)row * row_bytes, 0, 0);
                 }
     }
 }

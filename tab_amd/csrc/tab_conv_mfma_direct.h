@@ -58,6 +58,7 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
     constexpr int A_ITEMS = (A_GRANULES + kConvThreads - 1) / kConvThreads, B_ITEMS = (B_GRANULES + kConvThreads - 1) / kConvThreads;
     constexpr int BUF_DWORDS = 4 * (A_ITEMS + B_ITEMS) * kConvThreads;  // whole wave instructions
     constexpr int A_RUN = granule_run(PA, APL), B_RUN = granule_run(PB, BPL);
+    static_assert(BM % 64 == 0 && BN % 64 == 0, "one wave instruction moves 64 / RUN rows of one run");
 
     __shared__ __attribute__((aligned(16))) uint32_t lds[2 * BUF_DWORDS];
 
@@ -65,19 +66,21 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int r = lane & 31, kb = lane >> 5;
     const int wm = wave % WM, wn = wave / WM;
+    const int pixels = p.OH * p.OW;
+    const size_t image_words = (size_t)p.H * p.W * p.PC * APL;
+    const size_t filter_bytes = (size_t)p.G * BPL * 8;
+
     int tile_m, tile_n;
     if (!tile_of_workgroup(p, tile_m, tile_n)) return;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
     // ---- what this lane fetches: granule idx = tid + i * 256 = (run * ROWS + row) * RUN + column ------
-    const int pixels = p.OH * p.OW;
-    const int n_first = (int)div32((uint32_t)m0, p.div_pixels);  // uniform
-    const size_t image_words = (size_t)p.H * p.W * p.PC * APL;
-    const size_t a_bytes = (size_t)(p.N - n_first) * image_words * 8;
-    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)(p.qx + (size_t)n_first * image_words), 0, a_bytes > 0xffffffffull ? (int)0xffffffffu : (int)a_bytes, kBufferFlags);
     int ih0[A_ITEMS], iw0[A_ITEMS];
     uint32_t a_base[A_ITEMS], b_base[B_ITEMS];
+    const int n_first = (int)div32((uint32_t)m0, p.div_pixels);  // uniform
+    const size_t a_bytes = (size_t)(p.N - n_first) * image_words * 8;
+    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(p.qx + (size_t)n_first * image_words), 0,
+        a_bytes > 0xffffffffull ? (int)0xffffffffu : (int)a_bytes, kBufferFlags);
 #pragma unroll
     for (int i = 0; i < A_ITEMS; i++) {
         const int idx = tid + i * kConvThreads;
@@ -95,10 +98,9 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
         a_base[i] = (uint32_t)((((n - n_first) * p.H + (oh * p.s1 - p.p1)) * p.W + iw0[i]) * p.PC) * (uint32_t)(APL * 8) +
                     (uint32_t)in_run * 16u;
     }
-    const size_t filter_bytes = (size_t)p.G * BPL * 8;
     const size_t b_bytes = (size_t)(p.KN - n0) * filter_bytes;
-    const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)(p.qw + (size_t)n0 * p.G * BPL), 0, b_bytes > kNoFilter ? (int)kNoFilter : (int)b_bytes, kBufferFlags);
+    const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(p.qw + (size_t)n0 * p.G * BPL), 0,
+        b_bytes > kNoFilter ? (int)kNoFilter : (int)b_bytes, kBufferFlags);
 #pragma unroll
     for (int i = 0; i < B_ITEMS; i++) {
         const int idx = tid + i * kConvThreads;
@@ -107,9 +109,8 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
         const bool live = granule < PB && (n0 + row) < p.KN;
         b_base[i] = live ? (uint32_t)row * (uint32_t)filter_bytes + (uint32_t)granule * 16u : kNoFilter;
     }
-
-    static_assert(BM % 64 == 0 && BN % 64 == 0, "one wave instruction moves 64 / RUN rows of one run");
-    auto fetch = [&](int chunk, uint32_t *buf) {
+    // chunk `chunk` into buf; !live_chunk: zeros (every offset out of range)
+    auto fetch = [&](int chunk, uint32_t *buf, bool live_chunk) {
         const int g0 = chunk * KCH;  // first word of the chunk
 #pragma unroll
         for (int i = 0; i < A_ITEMS; i++) {
@@ -120,33 +121,19 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
             const int kh = (int)fastdiv(tap, p.div_kw);
             const int kw = (int)tap - kh * p.KW;
             const uint32_t tap_off = (uint32_t)((kh * p.W + kw) * p.PC + pc) * (uint32_t)(APL * 8);
-            const bool ok = (unsigned)(ih0[i] + kh) < (unsigned)p.H && (unsigned)(iw0[i] + kw) < (unsigned)p.W;
+            const bool ok = live_chunk && (unsigned)(ih0[i] + kh) < (unsigned)p.H && (unsigned)(iw0[i] + kw) < (unsigned)p.W;
             load16_to_lds(a_rsrc, buf + 4 * (i * kConvThreads + wave * 64), ok ? a_base[i] + tap_off : kNoData);
         }
         const uint32_t word_off = (uint32_t)g0 * (uint32_t)(BPL * 8);
 #pragma unroll
         for (int i = 0; i < B_ITEMS; i++)
             load16_to_lds(b_rsrc, buf + 4 * ((A_ITEMS + i) * kConvThreads + wave * 64),
-                          b_base[i] == kNoFilter ? kNoFilter : b_base[i] + word_off);
+                          b_base[i] == kNoFilter || !live_chunk ? kNoFilter : b_base[i] + word_off);
     };
 
     const ExpandConsts consts;
     f32x16 acc[TM][TN];
-#pragma unroll
-    for (int mt = 0; mt < TM; mt++)
-#pragma unroll
-        for (int nt = 0; nt < TN; nt++)
-#pragma unroll
-            for (int e = 0; e < 16; e++) acc[mt][nt][e] = 0.f;
     int b_nonzero[TN];
-#pragma unroll
-    for (int nt = 0; nt < TN; nt++) b_nonzero[nt] = 0;
-
-    const int wave_m0 = m0 + wm * (32 * TM), wave_n0 = n0 + wn * (32 * TN);
-
-    fetch(0, lds);
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
 
     // dword offset of this lane's part of a pair of words: one-plane: 8 bytes of the pair's granule; two-plane:
     // the granule of its own word, 2 * pair + kb.  Tile and wave offsets are multiples of 32 rows, so the
@@ -162,71 +149,152 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
     };
     constexpr int B_REGION = 4 * A_ITEMS * kConvThreads;
 
-    for (int chunk = 0; chunk < p.nchunks; chunk++) {
-        const bool more = chunk + 1 < p.nchunks;
-        if (more) fetch(chunk + 1, lds + ((chunk + 1) & 1) * BUF_DWORDS);
-
-        const uint32_t *buf = lds + (chunk & 1) * BUF_DWORDS;
-        uint32_t a_w[2][TM][2 * APL], b_w[2][TN][2 * BPL];  // [low half, high half] of every plane of the lane's word
-        auto read_pair = [&](int pair) {
+    constexpr int HS = TYPE == 5 ? 1 : 2;  // MFMA steps per pair of words: one per half, type 5 both halves at once
+    constexpr int STEPS = PAIRS * HS;
+    // (with one expansion or more per MFMA the vector unit is the limit either way and the pinned order only costs)
+    constexpr bool PIPELINED = TYPE != 5 && TM * TN >= 8;
+    constexpr int NM = TM * TN, NE = TM + TN;
+    uint32_t a_w[2][TM][2 * APL], b_w[2][TN][2 * BPL];  // [low half, high half] of every plane of the lane's word
+    auto read_pair = [&](const uint32_t *buf, int pair) {
 #pragma unroll
-            for (int mt = 0; mt < TM; mt++) {
-                const uint32_t *src = buf + lane_part(APL, A_RUN, BM, a_row, a_sw, pair) + mt * 32 * A_RUN * 4;
-                if (APL == 1) {
-                    const u32x2 v = *reinterpret_cast<const u32x2 *>(src);
-                    a_w[pair & 1][mt][0] = v[0]; a_w[pair & 1][mt][1] = v[1];
-                } else {
-                    const u32x4 v = *reinterpret_cast<const u32x4 *>(src);
+        for (int mt = 0; mt < TM; mt++) {
+            const uint32_t *src = buf + lane_part(APL, A_RUN, BM, a_row, a_sw, pair) + mt * 32 * A_RUN * 4;
+            if (APL == 1) {
+                const u32x2 v = *reinterpret_cast<const u32x2 *>(src);
+                a_w[pair & 1][mt][0] = v[0]; a_w[pair & 1][mt][1] = v[1];
+            } else {
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(src);
 #pragma unroll
-                    for (int e = 0; e < 4; e++) a_w[pair & 1][mt][e] = v[e];
-                }
-            }
-#pragma unroll
-            for (int nt = 0; nt < TN; nt++) {
-                const uint32_t *src = buf + B_REGION + lane_part(BPL, B_RUN, BN, b_row, b_sw, pair) + nt * 32 * B_RUN * 4;
-                if (BPL == 1) {
-                    const u32x2 v = *reinterpret_cast<const u32x2 *>(src);
-                    b_w[pair & 1][nt][0] = v[0]; b_w[pair & 1][nt][1] = v[1];
-                } else {
-                    const u32x4 v = *reinterpret_cast<const u32x4 *>(src);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) b_w[pair & 1][nt][e] = v[e];
-                }
-            }
-        };
-        read_pair(0);
-#pragma unroll
-        for (int pair = 0; pair < PAIRS; pair++) {
-            if (pair + 1 < PAIRS) read_pair(pair + 1);
-#pragma unroll
-            for (int h = 0; h < (TYPE == 5 ? 1 : 2); h++) {
-                i32x8 af[TM], bf[TN];
-#pragma unroll
-                for (int mt = 0; mt < TM; mt++) {
-                    const uint32_t *w = a_w[pair & 1][mt];
-                    af[mt] = TYPE == 5 ? expand_operand<TYPE, 0>(w[0], w[1], consts)
-                                       : expand_operand<TYPE, 0>(w[h], w[2 * (APL - 1) + h], consts);
-                }
-#pragma unroll
-                for (int nt = 0; nt < TN; nt++) {
-                    const uint32_t *w = b_w[pair & 1][nt];
-                    bf[nt] = TYPE == 5 ? expand_operand<TYPE, 1>(w[0], w[1], consts)
-                                       : expand_operand<TYPE, 1>(w[h], w[2 * (BPL - 1) + h], consts);
-                    if (TYPE == 2) b_nonzero[nt] += __builtin_popcount(w[2 + h]);
-                }
-#pragma unroll
-                for (int mt = 0; mt < TM; mt++)
-#pragma unroll
-                    for (int nt = 0; nt < TN; nt++)
-                        acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[mt], bf[nt], acc[mt][nt], 4, 4, 0, 0, 0, 0);
+                for (int e = 0; e < 4; e++) a_w[pair & 1][mt][e] = v[e];
             }
         }
+#pragma unroll
+        for (int nt = 0; nt < TN; nt++) {
+            const uint32_t *src = buf + B_REGION + lane_part(BPL, B_RUN, BN, b_row, b_sw, pair) + nt * 32 * B_RUN * 4;
+            if (BPL == 1) {
+                const u32x2 v = *reinterpret_cast<const u32x2 *>(src);
+                b_w[pair & 1][nt][0] = v[0]; b_w[pair & 1][nt][1] = v[1];
+            } else {
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(src);
+#pragma unroll
+                for (int e = 0; e < 4; e++) b_w[pair & 1][nt][e] = v[e];
+            }
+        }
+    };
+    // Software pipeline over the MFMA steps (PIPELINED): while the matrix cores work on step s the vector unit expands
+    // the operands of step s + 1 into the other set of operand registers, one operand after each MFMA (a wave issues in
+    // order: expansions written in front of their own MFMAs leave the matrix pipe idle meanwhile).  The raw words of a
+    // pair are read from LDS a step before their first expansion; those of the next chunk's first pair right after the
+    // barrier, which therefore stands before the chunk's last step.  The order is pinned with scheduling barriers: left
+    // alone, the scheduler sinks the LDS reads to their first use and the wave waits for LDS in the middle of the MFMAs.
+    i32x8 af[2][PIPELINED ? TM : 1], bf[2][PIPELINED ? TN : 1];
+    // operand e of a step, in the order the MFMAs need them: A0, B0 .. B(TN-1), A1 .. A(TM-1)
+    auto expand_one = [&](int e, int pair, int h, int set) {
+        if (e == 0 || e > TN) {
+            const int mt = e == 0 ? 0 : e - TN;
+            const uint32_t *w = a_w[pair & 1][mt];
+            af[set][mt] = expand_operand<TYPE, 0>(w[h], w[2 * (APL - 1) + h], consts);
+        } else {
+            const int nt = e - 1;
+            const uint32_t *w = b_w[pair & 1][nt];
+            bf[set][nt] = expand_operand<TYPE, 1>(w[h], w[2 * (BPL - 1) + h], consts);
+            if (TYPE == 2) b_nonzero[nt] += __builtin_popcount(w[2 + h]);  // (the zeros past the last chunk add nothing)
+        }
+    };
 
-        // keep the wait at the end of the chunk's MFMAs (the scheduler would hoist it above them, since
-        // only memory operations order it): the next chunk's loads have a whole chunk of work to land in
-        __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(0);  // this wave's part of the next chunk has landed
-        __syncthreads();
+    const int wave_m0 = m0 + wm * (32 * TM), wave_n0 = n0 + wn * (32 * TN);
+#pragma unroll
+    for (int mt = 0; mt < TM; mt++)
+#pragma unroll
+        for (int nt = 0; nt < TN; nt++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[mt][nt][e] = 0.f;
+#pragma unroll
+    for (int nt = 0; nt < TN; nt++) b_nonzero[nt] = 0;
+
+    fetch(0, lds, true);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if constexpr (PIPELINED) {
+        read_pair(lds, 0);
+#pragma unroll
+        for (int e = 0; e < NE; e++) expand_one(e, 0, 0, 0);
+    }
+
+    for (int chunk = 0; chunk < p.nchunks; chunk++) {
+        const bool more = chunk + 1 < p.nchunks;
+        const uint32_t *buf = lds + (chunk & 1) * BUF_DWORDS;
+        uint32_t *next = lds + ((chunk + 1) & 1) * BUF_DWORDS;
+
+        if constexpr (PIPELINED) {
+            // past the last chunk: zeros, which the last step expands and nobody uses
+            fetch(chunk + 1, next, more);
+#pragma unroll
+            for (int s = 0; s < STEPS; s++) {
+                const int pair = s / 2, h = s % 2;
+                const bool last = s == STEPS - 1;
+                __builtin_amdgcn_sched_barrier(0);
+                if (last) {
+                    __builtin_amdgcn_s_waitcnt(0);  // this wave's part of the next chunk has landed
+                    __syncthreads();
+                    read_pair(next, 0);
+                } else if (h == 0 && pair + 1 < PAIRS) {
+                    read_pair(buf, pair + 1);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                // the last step's expansions wait for the reads just issued: two MFMAs go first
+                const int delay = last ? 2 : 0;
+                const int per = (NE + (NM - delay) - 1) / (NM - delay);
+                const int npair = last ? 0 : (s + 1) / 2, nh = (s + 1) % 2;
+                int done = 0;
+#pragma unroll
+                for (int i = 0; i < NM; i++) {
+                    const int mt = i / TN, nt = i % TN;
+                    acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[s & 1][mt], bf[s & 1][nt], acc[mt][nt], 4, 4, 0, 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                    const int upto = i < delay ? 0 : ((i + 1 - delay) * per < NE ? (i + 1 - delay) * per : NE);
+#pragma unroll
+                    for (int e = 0; e < NE; e++)
+                        if (e >= done && e < upto) expand_one(e, npair, nh, (s + 1) & 1);
+                    done = upto;
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        } else {
+            if (more) fetch(chunk + 1, next, true);
+            read_pair(buf, 0);
+#pragma unroll
+            for (int pair = 0; pair < PAIRS; pair++) {
+                if (pair + 1 < PAIRS) read_pair(buf, pair + 1);
+#pragma unroll
+                for (int h = 0; h < HS; h++) {
+                    i32x8 a_op[TM], b_op[TN];
+#pragma unroll
+                    for (int mt = 0; mt < TM; mt++) {
+                        const uint32_t *w = a_w[pair & 1][mt];
+                        a_op[mt] = TYPE == 5 ? expand_operand<TYPE, 0>(w[0], w[1], consts)
+                                             : expand_operand<TYPE, 0>(w[h], w[2 * (APL - 1) + h], consts);
+                    }
+#pragma unroll
+                    for (int nt = 0; nt < TN; nt++) {
+                        const uint32_t *w = b_w[pair & 1][nt];
+                        b_op[nt] = TYPE == 5 ? expand_operand<TYPE, 1>(w[0], w[1], consts)
+                                             : expand_operand<TYPE, 1>(w[h], w[2 * (BPL - 1) + h], consts);
+                        if (TYPE == 2) b_nonzero[nt] += __builtin_popcount(w[2 + h]);
+                    }
+#pragma unroll
+                    for (int mt = 0; mt < TM; mt++)
+#pragma unroll
+                        for (int nt = 0; nt < TN; nt++)
+                            acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_op[mt], b_op[nt], acc[mt][nt], 4, 4, 0, 0, 0, 0);
+                }
+            }
+            // keep the wait at the end of the chunk's MFMAs (the scheduler would hoist it above them, since
+            // only memory operations order it): the next chunk's loads have a whole chunk of work to land in
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(0);  // this wave's part of the next chunk has landed
+            __syncthreads();
+        }
     }
 
     conv_mfma_epilogue<TYPE, TM, TN, KCH, 1>(p, acc, b_nonzero, wave_m0, wave_n0, lane, 0, nullptr);
