@@ -376,21 +376,28 @@ int conv_mfma_shape(int conv_type, const ConvArgs &a)
     if (conv_type <= 3 && a.G <= 9 && a.qy != nullptr && (a.M >= 65536 || a.G <= 2)) return 7;
     // short K: the per-tile prologue and epilogue weigh more, so a shape needs more tiles to pay
     const long enough = a.G >= 72 ? 192 : (a.G >= 36 ? 300 : 1024);
-    // eight tiles per wave share each expanded operand between more MFMAs (the dearer operand gets the
-    // 4-tile side): +2-18 %, but only when the launch is many rounds of these big tiles (512 run at a time), or,
-    // with long K and a two-plane operand (3-10 %), at least two rounds or most of a single one; in between the
-    // tail of the last round costs more than the shape gains
-    const long big_tiles = tiles(256, 128);
-    const bool rounds = a.G >= 36 && big_tiles >= 2560;
-    const bool long_k = type != 3 && a.G >= 72 && (big_tiles >= 1024 || (big_tiles >= 384 && big_tiles <= 512));
-    if (rounds || long_k) {
-        if (type == 1 && a.KN >= 256) return 6;
-        if (type != 1 && a.KN >= 128) return 5;
+    // eight tiles per wave share each expanded operand between more MFMAs, and their K loop is software-pipelined
+    // (expansions in the shadow of the MFMAs): per unit of work 3-12 % faster than the 128x128 shape, more the longer
+    // K is.  But a CU holds two such workgroups against four of the smaller shape, so what decides is the busiest
+    // CU: ceil(tiles / 256) tiles of either kind, the big ones twice the work each.  364 big tiles (two on some CUs)
+    // lose 5-12 % to 728 small ones (three), 392 (two) beat 784 (four) by 3-10 %, 784 lose again, 1456 win.  With K
+    // of 18 words only the types whose weights have two planes gained.  Which side gets four tiles: the dearer
+    // operand of TBN and BTN; TNN and, at long K, BNN measured 1-10 % faster with four filter tiles.
+    const long big_tiles = tiles(256, 128), small_tiles = tiles(128, 128);
+    const int unit_permille = a.G >= 72 ? 880 : (a.G >= 36 ? 920 : 970);  // time of a big tile / two small ones
+    // (packed output: its epilogue, a ballot per value, weighs more on eight tiles: only many rounds of them pay)
+    const bool eight = a.qy != nullptr ? a.G >= 36 && big_tiles >= 2560
+                                       : a.G >= (type == 0 || type == 2 ? 18 : 36) && big_tiles >= 160 &&
+                                             ((big_tiles + 255) / 256) * 2 * unit_permille < ((small_tiles + 255) / 256) * 1000;
+    if (eight) {
+        const bool wide = type == 1 || type == 0 || (type == 3 && a.G >= 72);
+        if (wide && a.KN >= 256) return 6;
+        if (a.KN >= 128) return 5;
     }
-    if (a.KN > 64 && tiles(128, 128) >= (a.G >= 18 ? enough : 4096)) return 0;
+    if (a.KN > 64 && tiles(128, 128) >= (a.G >= 18 ? enough : (type == 3 ? 4096 : 1536))) return 0;
     // one tile of filters: 256 rows per workgroup halve the expansions per MFMA of the 128x64 shape (two-plane
-    // operands gain 20 %, BNN nothing)
-    if (a.KN <= 64 && type != 3 && tiles(256, 64) >= 1024) return 4;
+    // operands gain 20 %, BNN 5-9 % on the largest launches only)
+    if (a.KN <= 64 && tiles(256, 64) >= (type != 3 ? 1024 : 4096)) return 4;
     // a handful of words of K (1x1 layers on few channels): the 64x64 shape's short prologue wins
     if (a.G <= 4 && tiles(64, 64) >= 192) return 2;
     if (tiles(128, 64) >= enough) return 1;
