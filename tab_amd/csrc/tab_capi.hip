@@ -243,6 +243,8 @@ static int conv_packed(const int64_t *dev_QX, const int64_t *dev_QW, const int32
     a.div_ow = tab::make_div32((uint32_t)s.OW);
     a.div_tiles_m = tab::make_div32(1);
     a.tiles_n = 0;
+    a.xcd_share = 0; a.filter_tiles = 1;
+    a.div_filter_tiles = tab::make_div32(1);
     hipError_t e = tab::launch_conv(type, a, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return device_fail(e, "conv launch");
     return TAB_OK;

@@ -103,6 +103,9 @@ def test_c_abi_rejects_bad_arguments_without_launching():
     # a packed image too large for 32-bit offsets inside one workgroup
     assert lib.tab_conv2d_packed(p, p, p, 3, 0, 0, 1, 1, 1, 30000, 30000, 64, 4, 1, 1, p, None) == -2
     assert b"32-bit" in lib.tab_last_error()
+    # a wave addresses its rows of Y with 32-bit byte offsets: 128 rows of KN floats stay below 2 GiB
+    assert lib.tab_conv2d_packed(p, p, p, 3, 0, 0, 1, 1, 1, 4, 4, 64, 1 << 22, 1, 1, p, None) == -2
+    assert b"KN" in lib.tab_last_error()
 
 
 def test_set_conv_kernel_validates_without_a_gpu():

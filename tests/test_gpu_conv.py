@@ -277,6 +277,18 @@ def test_short_k_large_output_workgroup_order(C, KN):
             assert bool(((y.to(torch.int64) - C) % 2 == 0).all())
 
 
+@pytest.mark.parametrize("C", [128, 64])  # the LDS-direct kernel and the register-staged one
+@pytest.mark.parametrize("type", [0, 3])
+def test_xcd_order_with_a_ragged_tile_count(type, C, restore_kernel_choice):
+    """Launches of 64 tiles and more hand each XCD an eighth of the tiles (workgroup b -> tile (b % 8) * share + b / 8)
+    and leave the last tiles % 8 where they are: every tile must still be computed exactly once.  M = 5 * 37 * 37 =
+    6845 rows and KN = 192 give 321 (64x64), 162 (128x64), 108 (128x128), 81 (256x64), 54 tiles (below 64: the plain
+    order) and 214 * 6 (32x32): counts that leave every remainder."""
+    for tile in (-1, 0, 1, 2, 3, 4, 5, 6):
+        tab_amd.set_conv_kernel(tab_amd.CONV_MATRIX if tile >= 0 else tab_amd.CONV_AUTO, tile)
+        _conv_case(type, 5, 37, 37, C, 192, 3, 3, 1, 1, 1, 1, seed=29 + tile)
+
+
 def test_conv_rejects_wrong_sizes():
     x = torch.zeros((1, 4, 4, 64), device="cuda")
     ths = torch.zeros(1, device="cuda")
