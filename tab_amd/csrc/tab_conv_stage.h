@@ -60,6 +60,7 @@ __device__ __forceinline__ void store_item(uint32_t *lds, const Item<PL> &it, in
             lds[((pl * Q) + 2 * word + half) * ROWS + row] = it.d[pl * 2 + half];
 }
 
+constexpr int kStreamingStore = 2;  // cache policy of a buffer store: non-temporal (the nt bit)
 constexpr uint32_t kNoData = 0xffffffffu;     // activation offset that is always out of range
 constexpr uint32_t kNoFilter = 0x80000000u;   // weight offsets stay below this; adding it leaves the range
 
