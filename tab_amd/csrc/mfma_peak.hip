@@ -3,7 +3,11 @@
 // all four operand combinations, (2) measures the instruction's issue rate alone and with the
 // per-tile expansion work of each conv type in front of it, for the tiles per wave and workgroups per CU the conv
 // kernel runs (2x2 at up to four workgroups, 4x2 / 2x4 at two), (3) measures how many independent vector
-// instructions fit in an MFMA's shadow.  Register-resident: no memory traffic in the timed loops.
+// instructions fit in an MFMA's shadow, (4) compares the two orders of a step of the conv kernel's loop: all
+// expansions, then the MFMAs (serial), against the next step's expansions one after each MFMA of this step
+// into a second set of operand registers (pipelined), with the expansion constants in registers as in the
+// kernel, and reports the shader clock each run held (s_memtime over s_memrealtime).
+// Register-resident: no memory traffic in the timed loops.
 #include <hip/hip_runtime.h>
 #include <cstdio>
 #include <cstdint>
@@ -134,6 +138,90 @@ template <int NV> int shadow(int bpc)
     CK(hipFree(out));
     return 0;
 }
+
+// The conv kernel's expansions with their constants in registers (mask in an SGPR, patterns in VGPRs): 7 vector
+// instructions for a binary operand, 12 for a ternary one.
+struct ExpandRegs { uint32_t m3, p0, p1, p2, m0, m1, m2; };
+__device__ __forceinline__ ExpandRegs expand_regs()
+{
+    ExpandRegs k = {M3, M0, M1, M2, M0, M1, M2};
+    asm volatile("" : "+s"(k.m3), "+s"(k.m0), "+s"(k.m1), "+s"(k.m2));
+    asm volatile("" : "+v"(k.p0), "+v"(k.p1), "+v"(k.p2));
+    return k;
+}
+__device__ __forceinline__ v8i bin_regs(uint32_t w, const ExpandRegs &k)
+{
+    v8i r = {0, 0, 0, 0, 0, 0, 0, 0};
+    r[0] = (int)(((w << 3) & k.m3) | k.p0); r[1] = (int)(((w << 2) & k.m3) | k.p1); r[2] = (int)(((w << 1) & k.m3) | k.p2); r[3] = (int)((w & k.m3) | k.p2);
+    return r;
+}
+__device__ __forceinline__ v8i ter_regs(uint32_t s, uint32_t z, const ExpandRegs &k)
+{
+    v8i r = {0, 0, 0, 0, 0, 0, 0, 0};
+    r[0] = (int)((z & k.m0) | ((s << 3) & k.m3)); r[1] = (int)((z & k.m1) | ((s << 2) & k.m3));
+    r[2] = (int)((z & k.m2) | ((s << 1) & k.m3)); r[3] = (int)(((z >> 1) & k.m2) | (s & k.m3));
+    return r;
+}
+// TER: ternary operands on both sides.  PIPE 0: the TM + TN expansions of a step, then its TM * TN MFMAs; 1: the
+// MFMAs of a step with the next step's expansions one after each, into the other operand set.  Order pinned.
+template <int TER, int PIPE, int TM, int TN>
+__global__ __launch_bounds__(256) void k_step_order(float *out, long long *clocks, int iters, uint32_t seed)
+{
+    constexpr int NE = TM + TN, NM = TM * TN;
+    v16f c[TM][TN];
+    for (int i = 0; i < TM; i++) for (int j = 0; j < TN; j++) for (int e = 0; e < 16; e++) c[i][j][e] = 0;
+    uint32_t w[2 * NE];
+    for (int i = 0; i < 2 * NE; i++) w[i] = seed * (threadIdx.x + 1) * (2 * i + 1);
+    const ExpandRegs k = expand_regs();
+    v8i op[2][NE];
+    for (int e = 0; e < NE; e++) op[0][e] = op[1][e] = bin_regs(w[e], k);
+    const long long t0 = clock64(), r0 = wall_clock64();
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            if (PIPE == 0) {
+#pragma unroll
+                for (int e = 0; e < NE; e++) op[s][e] = TER ? ter_regs(w[e], w[NE + e], k) : bin_regs(w[e], k);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < NM; i++) c[i / TN][i % TN] = mfma(op[s][i / TN], op[s][TM + i % TN], c[i / TN][i % TN]);
+                __builtin_amdgcn_sched_barrier(0);
+            } else {
+#pragma unroll
+                for (int i = 0; i < NM; i++) {
+                    c[i / TN][i % TN] = mfma(op[s][i / TN], op[s][TM + i % TN], c[i / TN][i % TN]);
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (i < NE) op[s ^ 1][i] = TER ? ter_regs(w[i], w[NE + i], k) : bin_regs(w[i], k);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            w[0] += 0x9e3779b9u; for (int i = 1; i < 2 * NE; i++) w[i] ^= w[i - 1];  // new raw words every step
+        }
+    }
+    const long long t1 = clock64(), r1 = wall_clock64();
+    if (blockIdx.x == 0 && threadIdx.x == 0) { clocks[0] = t1 - t0; clocks[1] = r1 - r0; }
+    float sum = 0;
+    for (int i = 0; i < TM; i++) for (int j = 0; j < TN; j++) for (int e = 0; e < 16; e++) sum += c[i][j][e];
+    if (sum == 12345.678f) out[threadIdx.x] = sum;
+}
+template <int TER, int PIPE, int TM, int TN> int step_order(int bpc)
+{
+    float *out; long long *clocks, h[2];
+    CK(hipMalloc(&out, 4096)); CK(hipMalloc(&clocks, 16));
+    const int iters = 2000, blocks = 256 * bpc;
+    hipEvent_t e0, e1; CK(hipEventCreate(&e0)); CK(hipEventCreate(&e1));
+    k_step_order<TER, PIPE, TM, TN><<<blocks, 256>>>(out, clocks, 10, 3); CK(hipDeviceSynchronize());
+    CK(hipEventRecord(e0)); k_step_order<TER, PIPE, TM, TN><<<blocks, 256>>>(out, clocks, iters, 3); CK(hipEventRecord(e1)); CK(hipEventSynchronize(e1));
+    float ms; CK(hipEventElapsedTime(&ms, e0, e1));
+    CK(hipMemcpy(h, clocks, 16, hipMemcpyDeviceToHost));
+    const double mhz = (double)h[0] / ((double)h[1] / 100.0);  // s_memrealtime ticks at 100 MHz
+    const double per_simd = (double)bpc * iters * 2 * TM * TN;
+    printf("%s operands, %s step, tiles/wave=%dx%d blocks/CU=%d: %.3f ms, shader clock %.0f MHz, cycles per MFMA per SIMD at that clock = %.1f, %.0f binary-equivalent TOP/s\n",
+           TER ? "ternary" : "binary ", PIPE ? "pipelined" : "serial   ", TM, TN, bpc, ms, mhz, ms * 1e-3 * mhz * 1e6 / per_simd,
+           2.0 * 256 * 4 * per_simd * 32 * 32 * 64 / (ms * 1e-3) / 1e12);
+    CK(hipFree(out)); CK(hipFree(clocks));
+    return 0;
+}
 static int val_t(uint32_t s, uint32_t z, int k) { return ((z >> k) & 1) ? (((s >> k) & 1) ? -1 : 1) : 0; }
 static int val_b(uint32_t w, int k) { return ((w >> k) & 1) ? -1 : 1; }
 int main()
@@ -169,5 +257,7 @@ int main()
         tput<1, 4, 2>("BNN expansions", bpc); tput<3, 2, 4>("TBN expansions", bpc); tput<2, 4, 2>("TNN expansions", bpc);
     }
     for (int bpc : {2, 4}) { shadow<0>(bpc); shadow<1>(bpc); shadow<2>(bpc); shadow<3>(bpc); shadow<4>(bpc); shadow<6>(bpc); }
+    for (int bpc : {1, 2}) { step_order<0, 0, 4, 2>(bpc); step_order<0, 1, 4, 2>(bpc); step_order<1, 0, 4, 2>(bpc); step_order<1, 1, 4, 2>(bpc); }
+    step_order<0, 0, 2, 2>(4); step_order<0, 1, 2, 2>(4); step_order<1, 0, 2, 2>(4); step_order<1, 1, 2, 2>(4);
     return 0;
 }
