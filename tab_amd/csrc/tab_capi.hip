@@ -244,6 +244,12 @@ static int conv_packed(const int64_t *dev_QX, const int64_t *dev_QW, const int32
     a.div_tiles_m = tab::make_div32(1);
     a.tiles_n = 0;
     a.xcd_share = 0; a.filter_tiles = 1;
+    // A Y that fits the 256 MB last-level cache beside the operands but not the L2s is written through the caches
+    // (the cache takes the stores faster than HBM: Y of 190-206 MB 1-11 % sooner); every other Y with non-temporal
+    // stores: a smaller one leaves no dirty L2 to flush when the launch ends (7-25 % sooner), a larger one would only
+    // push the operands out (Y of 411 MB: 7-28 % sooner).  At 103 MB the two policies measured within 3 %.
+    const long y_bytes = s.M * (long)KN * 4;
+    a.y_cached = y_bytes >= (128L << 20) && y_bytes <= (240L << 20);
     a.div_filter_tiles = tab::make_div32(1);
     hipError_t e = tab::launch_conv(type, a, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return device_fail(e, "conv launch");

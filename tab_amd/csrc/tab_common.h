@@ -70,6 +70,7 @@ struct ConvArgs {
     int tiles_m;   // ceil(M / BM)
     int tiles_n;   // filter tiles when the workgroups are ordered by rows of Y (LDS-direct kernel, short K), else 0
     Div32 div_tiles_m;  // by tiles_m, or by 8 * tiles_n in that order (set by the launchers)
+    int y_cached;       // fp32 output through the caches (1) or with non-temporal stores (0)
     int xcd_share;      // tiles each of the 8 XCDs takes as one contiguous run of rows of Y (0: order not XCD-aware)
     int filter_tiles;   // ceil(KN / BN), with div_filter_tiles, for that order
     Div32 div_filter_tiles;

@@ -246,7 +246,8 @@ __device__ __forceinline__ void conv_mfma_epilogue(const ConvArgs &p, f32x16 (&a
         return;
     }
     // Y is written once and read by nobody here: non-temporal stores keep it from pushing the operands out of L2
-    // (N=256 28x28x512->512: HBM reads 30-78 MB -> 15-31 MB, 1.1-1.3 x the operands' size, and 2-4 % less time).
+    // (N=256 28x28x512->512: HBM reads 30-78 MB -> 15-31 MB, 1.1-1.3 x the operands' size, and 2-4 % less time);
+    // p.y_cached (set from the size of Y by the host) selects ordinary stores instead.
     // fp32 output through a buffer descriptor over the wave's rows of Y: rows past M lie past its end and
     // columns past KN get an offset past it, so every store is unconditional (a branch per store, which
     // "if (in range) store" compiles to, cost more than the store: the epilogue of a 256x128 tile took 6.5 us)
@@ -266,16 +267,20 @@ __device__ __forceinline__ void conv_mfma_epilogue(const ConvArgs &p, f32x16 (&a
         if (TYPE == 3) bias = (float)(p.num - 64 * p.nchunks * KCH);
         // kNoFilter + any offset inside the tile stays out of range without wrapping
         const uint32_t lane_off = col < p.KN ? (uint32_t)(4 * kb) * row_bytes + (uint32_t)col * 4u : kNoFilter;
+        auto store_tiles = [&](auto policy) {
 #pragma unroll
-        for (int mt = 0; mt < TM; mt++)
+            for (int mt = 0; mt < TM; mt++)
 #pragma unroll
-            for (int j = 0; j < 4; j++)
+                for (int j = 0; j < 4; j++)
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int row = mt * 32 + 8 * j + i;  // + 4*kb, already in lane_off
-                    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[mt][nt][4 * j + i] + bias), y_rsrc,
-                                                          lane_off + (uint32_t)row * row_bytes, 0, kStreamingStore);
-                }
+                    for (int i = 0; i < 4; i++) {
+                        const int row = mt * 32 + 8 * j + i;  // + 4*kb, already in lane_off
+                        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[mt][nt][4 * j + i] + bias), y_rsrc,
+                                                              lane_off + (uint32_t)row * row_bytes, 0, decltype(policy)::value);
+                    }
+        };
+        if (p.y_cached) store_tiles(std::integral_constant<int, 0>());  // wave-uniform
+        else store_tiles(std::integral_constant<int, kStreamingStore>());
     }
 }
 
