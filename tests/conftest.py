@@ -22,3 +22,16 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture(autouse=True)
+def _automatic_conv_kernel_after_every_test():
+    """The kernel choice of tab_set_conv_kernel is process-wide: whatever a test selected (and however it ended),
+    the next test starts from the library's own choice."""
+    yield
+    try:
+        from tab_amd import _capi
+        lib = _capi.load()
+    except Exception:  # library not built: the tests that need it fail on their own
+        return
+    lib.tab_set_conv_kernel(0, -1)
