@@ -385,10 +385,12 @@ int conv_mfma_shape(int conv_type, const ConvArgs &a)
     // operand of TBN and BTN; TNN and, at long K, BNN measured 1-10 % faster with four filter tiles.
     const long big_tiles = tiles(256, 128), small_tiles = tiles(128, 128);
     const int unit_permille = a.G >= 72 ? 880 : (a.G >= 36 ? 920 : 970);  // time of a big tile / two small ones
-    // (packed output: its epilogue, a ballot per value, weighs more on eight tiles: only many rounds of them pay)
-    const bool eight = a.qy != nullptr ? a.G >= 36 && big_tiles >= 2560
-                                       : a.G >= (type == 0 || type == 2 ? 18 : 36) && big_tiles >= 160 &&
-                                             ((big_tiles + 255) / 256) * 2 * unit_permille < ((small_tiles + 255) / 256) * 1000;
+    // (packed output from the register-staged kernel, PC odd: its epilogue, a ballot per value, weighs more on eight
+    // tiles, and only many rounds of them pay)
+    const bool eight = a.qy != nullptr && a.PC % 2 != 0
+                           ? a.G >= 36 && big_tiles >= 2560
+                           : a.G >= (type == 0 || type == 2 ? 18 : 36) && big_tiles >= 160 &&
+                                 ((big_tiles + 255) / 256) * 2 * unit_permille < ((small_tiles + 255) / 256) * 1000;
     if (eight) {
         const bool wide = type == 1 || type == 0 || (type == 3 && a.G >= 72);
         if (wide && a.KN >= 256) return 6;

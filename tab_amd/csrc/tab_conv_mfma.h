@@ -127,7 +127,7 @@ __device__ __forceinline__ i32x8 expand_operand(uint32_t p0, uint32_t p1, const 
 // C[8*j + 4*kb + i][r] of the wave's 32x32 tile (mt, nt).  b_nonzero: BTN, bits set in the nonzero plane of
 // the k-positions this lane multiplied, per filter tile; partial: KS * 17 * 64 floats of LDS when the KS
 // waves of the workgroup hold partial sums of one tile.
-template <int TYPE, int TM, int TN, int KCH, int KS>
+template <int TYPE, int TM, int TN, int KCH, int KS, bool BALLOT_PACKING = true>
 __device__ __forceinline__ void conv_mfma_epilogue(const ConvArgs &p, f32x16 (&acc)[TM][TN], int (&b_nonzero)[TN], int wave_m0,
                                                    int wave_n0, int lane, int ks, float *partial)
 {
@@ -145,7 +145,7 @@ __device__ __forceinline__ void conv_mfma_epilogue(const ConvArgs &p, f32x16 (&a
 #pragma unroll
     for (int mt = 0; mt < TM; mt++) {
         th_row[mt] = 0.f;
-        if (p.qy != nullptr) {
+        if (BALLOT_PACKING && p.qy != nullptr) {
             int n = (int)div32((uint32_t)(wave_m0 + mt * 32 + r), p.div_pixels);
             n = n < p.N ? n : p.N - 1;  // rows past M are computed but not stored
             th_row[mt] = p.out_ths[n];
@@ -178,7 +178,7 @@ __device__ __forceinline__ void conv_mfma_epilogue(const ConvArgs &p, f32x16 (&a
         }
         return;
     }
-    if (p.qy != nullptr) {
+    if (BALLOT_PACKING && p.qy != nullptr) {
         // Packed output: Y is not written; each value is thresholded like the quantizer would
         // threshold it as the next layer's NHWC activation (item = image, channel = filter;
         // TAB_GEMM.cu:184-192, 231) and a wave ballot is 32 channels of two output pixels: lanes
@@ -282,6 +282,109 @@ __device__ __forceinline__ void conv_mfma_epilogue(const ConvArgs &p, f32x16 (&a
         if (p.y_cached) store_tiles(std::integral_constant<int, 0>());  // wave-uniform
         else store_tiles(std::integral_constant<int, kStreamingStore>());
     }
+}
+
+// Packed output for a kernel that multiplied with the weights as the FIRST MFMA operand: accumulator element 4j+i of
+// lane (kb, r) is then filter 8j+4kb+i of filter tile nt and pixel r of row tile mt, i.e. a lane holds 16 filters of ONE
+// pixel.  It thresholds them against that pixel's threshold (a per-lane constant) exactly as the quantizer would
+// threshold them as the next layer's NHWC activation (item = image, channel = filter; TAB_GEMM.cu:184-192, 231) into 16
+// bits, and the other half-wave's lane of the same pixel supplies the other 16 of the 32-bit half word: no ballot and
+// no cross-lane deposit per value (the ballot form above costs about 13 vector instructions per pair of rows, this
+// one 2-3 per value).  The per-filter bias of BTN (btn - nonzero weights, known per lane = filter after the loop) is
+// handed to the lanes that need it through `exchange`, 32*TN dwords of LDS private to the wave.
+template <int TYPE, int TM, int TN, int KCH>
+__device__ __forceinline__ void conv_mfma_epilogue_packed(const ConvArgs &p, f32x16 (&acc)[TM][TN], int (&b_nonzero)[TN], int wave_m0,
+                                                          int wave_n0, int lane, uint32_t *exchange)
+{
+    const int r = lane & 31, kb = lane >> 5;
+    const long rows_left = (long)p.M - wave_m0;
+    if (rows_left <= 0) return;  // wave-uniform
+    const int out_words = (p.KN + 63) >> 6;
+    const uint32_t element = p.out_bits == 1 ? 8u : 16u;
+    const uint32_t row_bytes = (uint32_t)out_words * element;
+    const __amdgpu_buffer_rsrc_t out = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(reinterpret_cast<char *>(p.qy) + (size_t)wave_m0 * row_bytes), 0,
+        (int)((uint32_t)(rows_left < 32 * TM ? rows_left : 32 * TM) * row_bytes), kBufferFlags);
+
+    float bias[TN][16];
+#pragma unroll
+    for (int nt = 0; nt < TN; nt++) {
+        if (TYPE == 2) {
+            const int col = wave_n0 + nt * 32 + r;
+            const int btn = col < p.KN ? p.btn[col] : 0;
+            const int nonzero = b_nonzero[nt] + __shfl_xor(b_nonzero[nt], 32, 64);
+            exchange[nt * 32 + r] = __float_as_uint((float)(btn - nonzero));  // both half-waves write the same value
+        }
+    }
+    if (TYPE == 2) __builtin_amdgcn_wave_barrier();  // LDS operations of one wave complete in order
+#pragma unroll
+    for (int nt = 0; nt < TN; nt++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            u32x4 v = {0, 0, 0, 0};
+            if (TYPE == 2) v = *reinterpret_cast<const u32x4 *>(exchange + nt * 32 + 8 * j + 4 * kb);
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                bias[nt][4 * j + i] = TYPE == 2 ? __uint_as_float(v[i]) : (TYPE == 3 ? (float)(p.num - 64 * p.nchunks * KCH) : 0.f);
+        }
+
+    auto pack_rows = [&](auto out_bits_constant) {
+        constexpr int OUT_BITS = decltype(out_bits_constant)::value;
+#pragma unroll
+        for (int mt = 0; mt < TM; mt++) {
+            int n = (int)div32((uint32_t)(wave_m0 + mt * 32 + r), p.div_pixels);
+            n = n < p.N ? n : p.N - 1;  // rows past M are computed but not stored
+            const float th = p.out_ths[n];
+            uint32_t sign_half[TN], nz_half[TN];
+#pragma unroll
+            for (int nt = 0; nt < TN; nt++) {
+                uint32_t sg = 0, nz = 0;
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const float v = (TYPE == 2 || TYPE == 3) ? acc[mt][nt][4 * j + i] + bias[nt][4 * j + i] : acc[mt][nt][4 * j + i];
+                        const uint32_t bit = 1u << (8 * j + i);  // shifted by 4*kb below
+                        if (OUT_BITS == 1) {
+                            sg |= v < th ? bit : 0u;
+                        } else {
+                            const bool pos = v > th, neg = !pos && v < -th;
+                            sg |= neg ? bit : 0u;
+                            nz |= (pos || neg) ? bit : 0u;
+                        }
+                    }
+                const int cols_left = p.KN - (wave_n0 + nt * 32);  // filters of this tile that exist: tail bits stay zero
+                const uint32_t live = cols_left >= 32 ? 0xffffffffu : (cols_left <= 0 ? 0u : (1u << cols_left) - 1u);
+                sg <<= 4 * kb;
+                nz <<= 4 * kb;
+                sign_half[nt] = (sg | (uint32_t)__shfl_xor((int)sg, 32, 64)) & live;
+                nz_half[nt] = (nz | (uint32_t)__shfl_xor((int)nz, 32, 64)) & live;
+            }
+            // the lower half-wave stores; a word past the last one and the upper half-wave get an offset out of range
+            const uint32_t row_off = (uint32_t)(mt * 32 + r) * row_bytes;
+            if constexpr (TN % 2 == 0) {  // wave_n0 is a multiple of 64: tiles 2t, 2t+1 are the halves of one word
+#pragma unroll
+                for (int t = 0; t < TN / 2; t++) {
+                    const int word = (wave_n0 >> 6) + t;
+                    const uint32_t off = (kb == 0 && word < out_words) ? row_off + (uint32_t)word * element : kNoData;
+                    if (OUT_BITS == 1)
+                        __builtin_amdgcn_raw_buffer_store_b64(u32x2{sign_half[2 * t], sign_half[2 * t + 1]}, out, off, 0, 0);
+                    else
+                        __builtin_amdgcn_raw_buffer_store_b128(u32x4{sign_half[2 * t], sign_half[2 * t + 1], nz_half[2 * t], nz_half[2 * t + 1]}, out, off, 0, 0);
+                }
+            } else {
+#pragma unroll
+                for (int nt = 0; nt < TN; nt++) {
+                    const int col0 = wave_n0 + nt * 32, word = col0 >> 6, half = (col0 >> 5) & 1;
+                    const uint32_t off = (kb == 0 && word < out_words) ? row_off + (uint32_t)word * element + (uint32_t)half * 4u : kNoData;
+                    __builtin_amdgcn_raw_buffer_store_b32(sign_half[nt], out, off, 0, 0);
+                    if (OUT_BITS == 2) __builtin_amdgcn_raw_buffer_store_b32(nz_half[nt], out, off == kNoData ? kNoData : off + 8u, 0, 0);
+                }
+            }
+        }
+    };
+    if (p.out_bits == 1) pack_rows(std::integral_constant<int, 1>());  // wave-uniform
+    else pack_rows(std::integral_constant<int, 2>());
 }
 
 // Workgroup -> tile.  Small launches: the row tiles of one filter tile first.  From 64 tiles on: each XCD an eighth

@@ -46,7 +46,8 @@ __device__ __forceinline__ int run_swizzle(int row)
     return RUN == 4 ? ((row >> 1) + (row >> 3)) & 3 : (RUN == 2 ? ((row >> 2) + (row >> 3)) & 1 : 0);
 }
 
-template <int TYPE, int WM, int WN, int TM, int TN, int KCH>
+// PACKED: packed output (p.qy): the weights are the first MFMA operand and the epilogue packs inside a lane.
+template <int TYPE, int WM, int WN, int TM, int TN, int KCH, bool PACKED>
 __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM * TN > 4 ? 2 : (WM * TM > 4 ? 3 : 4)))) void conv_mfma_direct(const ConvArgs p)
 {
     static_assert(WM * WN * 64 == kConvThreads && KCH % 2 == 0, "four waves, whole pairs of words");
@@ -250,7 +251,8 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
 #pragma unroll
                 for (int i = 0; i < NM; i++) {
                     const int mt = i / TN, nt = i % TN;
-                    acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[s & 1][mt], bf[s & 1][nt], acc[mt][nt], 4, 4, 0, 0, 0, 0);
+                    acc[mt][nt] = PACKED ? __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[s & 1][nt], af[s & 1][mt], acc[mt][nt], 4, 4, 0, 0, 0, 0)
+                                         : __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[s & 1][mt], bf[s & 1][nt], acc[mt][nt], 4, 4, 0, 0, 0, 0);
                     __builtin_amdgcn_sched_barrier(0);
                     const int upto = i < delay ? 0 : ((i + 1 - delay) * per < NE ? (i + 1 - delay) * per : NE);
 #pragma unroll
@@ -286,7 +288,8 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
                     for (int mt = 0; mt < TM; mt++)
 #pragma unroll
                         for (int nt = 0; nt < TN; nt++)
-                            acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_op[mt], b_op[nt], acc[mt][nt], 4, 4, 0, 0, 0, 0);
+                            acc[mt][nt] = PACKED ? __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b_op[nt], a_op[mt], acc[mt][nt], 4, 4, 0, 0, 0, 0)
+                                             : __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_op[mt], b_op[nt], acc[mt][nt], 4, 4, 0, 0, 0, 0);
                 }
             }
             // keep the wait at the end of the chunk's MFMAs (the scheduler would hoist it above them, since
@@ -297,7 +300,12 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
         }
     }
 
-    conv_mfma_epilogue<TYPE, TM, TN, KCH, 1>(p, acc, b_nonzero, wave_m0, wave_n0, lane, 0, nullptr);
+    if constexpr (PACKED) {
+        // (a wave that is still in its last step only reads operands nobody uses any more)
+        conv_mfma_epilogue_packed<TYPE, TM, TN, KCH>(p, acc, b_nonzero, wave_m0, wave_n0, lane, lds + wave * (32 * TN));
+    } else {
+        conv_mfma_epilogue<TYPE, TM, TN, KCH, 1, false>(p, acc, b_nonzero, wave_m0, wave_n0, lane, 0, nullptr);
+    }
 }
 
 template <int TYPE, int WM, int WN, int TM, int TN, int KCH>
@@ -312,7 +320,14 @@ hipError_t launch_mfma_direct(ConvArgs a, hipStream_t stream)
     a.tiles_m = (a.M + BM - 1) / BM;
     const long blocks = order_workgroups<Planes<TYPE>::A>(a, (a.KN + BN - 1) / BN);
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
-    conv_mfma_direct<TYPE, WM, WN, TM, TN, KCH><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
+    if (a.qy != nullptr) {
+        if constexpr (TYPE <= 3)
+            conv_mfma_direct<TYPE, WM, WN, TM, TN, KCH, true><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
+        else
+            return hipErrorInvalidValue;  // no packed output for types 4 and 5
+    } else {
+        conv_mfma_direct<TYPE, WM, WN, TM, TN, KCH, false><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
+    }
     return hipGetLastError();
 }
 

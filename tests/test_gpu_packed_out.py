@@ -66,11 +66,14 @@ def test_packed_out(type, case, out_bits):
 
 
 @pytest.mark.parametrize("tile", [0, 1, 2, 4, 5, 6, 7])
-@pytest.mark.parametrize("type", [0, 3])
+@pytest.mark.parametrize("type", [0, 1, 2, 3])
 def test_packed_out_every_tile(type, tile, restore_kernel_choice):
+    """Every shape packs its output: C = 192 and 256 take the kernel that multiplies with the weights first and packs
+    inside a lane (BTN hands its per-filter bias round through LDS there), C = 70 the one that packs by ballot."""
     tab_amd.set_conv_kernel(tab_amd.CONV_MATRIX, tile)
-    for case in (CASES[2], CASES[3], (1, 28, 28, 256, 256, 3, 3, 1, 1, 1, 1)):
-        _packed_out_case(type, *case, 2 - (type == 3), "integer", seed=9)
+    for out_bits in (1, 2):
+        for case in (CASES[1], CASES[2], CASES[3], (1, 28, 28, 256, 256, 3, 3, 1, 1, 1, 1)):
+            _packed_out_case(type, *case, out_bits, "integer", seed=9 + out_bits)
 
 
 def test_packed_out_ignores_popcount_choice(restore_kernel_choice):
