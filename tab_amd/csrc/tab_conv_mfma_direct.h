@@ -301,7 +301,9 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
     }
 
     if constexpr (PACKED) {
-        // (a wave that is still in its last step only reads operands nobody uses any more)
+        // BTN hands its biases round through LDS: not before every wave has read its last operands (the pipelined
+        // loop reads the zeros past the last chunk after the chunk's barrier and counts their nonzero weights)
+        if (TYPE == 2) __syncthreads();
         conv_mfma_epilogue_packed<TYPE, TM, TN, KCH>(p, acc, b_nonzero, wave_m0, wave_n0, lane, lds + wave * (32 * TN));
     } else {
         conv_mfma_epilogue<TYPE, TM, TN, KCH, 1, false>(p, acc, b_nonzero, wave_m0, wave_n0, lane, 0, nullptr);
