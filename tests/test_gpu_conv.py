@@ -103,6 +103,8 @@ VARIANT_CASES = [
     (2, 9, 9, 512, 72, 3, 3, 1, 1, 2, 2),      # PC = 8: chunks of four words inside a tap
     (1, 3, 3, 8192, 12, 3, 3, 1, 1, 1, 1),     # K = 73728 bits
     (2, 10, 10, 384, 136, 3, 3, 1, 1, 1, 1),   # PC = 6: six-word chunks across taps in every tile shape
+    (2, 9, 9, 256, 72, 1, 1, 0, 0, 1, 1),      # K = one chunk of four words: a pipelined loop's prologue meets its last step
+    (3, 7, 7, 128, 40, 1, 1, 0, 0, 1, 1),      # K = one chunk of two words (two MFMA steps)
 ]
 
 
