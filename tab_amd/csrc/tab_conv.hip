@@ -13,6 +13,7 @@
 // one k-slice with 128-bit LDS reads (A reads broadcast over the 16 tx lanes, B reads are
 // 256 B contiguous per 16 lanes).  The inner loop is pure VALU: XOR/AND + v_bcnt_u32_b32
 // with the count accumulated in the instruction's addend.
+#include "tab_conv_shape_model.h"
 #include "tab_conv_stage.h"
 
 #include <atomic>
@@ -360,51 +361,46 @@ hipError_t launch_conv_mfma(int type, const ConvArgs &args, int shape, hipStream
     }
 }
 
-// Workgroup tile of the matrix-core kernel, from measurements over the ResNet-18, VGG and sweep layers at
-// N = 8 .. 256: the 128-row tiles win as soon as there is about one of them per CU (with short K the
-// 128x128 one needs several per CU); below roughly 200 workgroups of 64x64 the launch is latency-bound
-// and the k-split 32x32 shape wins.
+// Workgroup tile of the matrix-core kernel: the shape with the lowest predicted duration under a cost model fitted to
+// the measured duration of every shape on 280 (type, layer) cases (tab_conv_shape_model.h: the ResNet-18 layers at
+// N = 16 / 64 / 256, the VGG stack, the 28x28 sweep and layers of other geometries).  What the model's features say:
+// the busiest of the 256 CUs decides (ceil(tiles / 256) tiles of a shape land on it, and it is refilled when it holds
+// no more), K scales the loop, the size of Y the epilogue, and a launch smaller than the chip is as long as one tile.
+// A shape whose filter tile is at least twice the 64-rounded filter count is no candidate.  Regret of the choice
+// against the best measured shape: 1.5 % over the fitted cases, 2.3 % with each layer set held out of the fit in turn
+// (the thresholds this replaces: 2.8 % on the same measurements, 5.5 % on the geometries they were not made from).
 int conv_mfma_shape(int conv_type, const ConvArgs &a)
 {
     // the CPU-only types follow the type with the same planes: 4 like TNN, 5 like BNN
     const int type = conv_type == 4 ? 0 : (conv_type == 5 ? 3 : conv_type);
-    auto tiles = [&](int bm, int bn) { return (long)((a.M + bm - 1) / bm) * ((a.KN + bn - 1) / bn); };
     // K of at most nine words and packed output: the kernel with the weights resident in registers, whose epilogue
     // thresholds a pixel's filters inside a lane, runs 1.4-2x faster than the tiled shapes once the launch is a few
     // rounds of waves (N=256 56x56x64->64 3x3: 24 against 38 us) and level with them on small ones; with fp32 output
     // both are bound by writing Y and measure within 5 % of each other, so the tiled shapes keep those launches
     if (conv_type <= 3 && a.G <= 9 && a.qy != nullptr && (a.M >= 65536 || a.G <= 2)) return 7;
-    // short K: the per-tile prologue and epilogue weigh more, so a shape needs more tiles to pay
-    const long enough = a.G >= 72 ? 192 : (a.G >= 36 ? 300 : 1024);
-    // eight tiles per wave share each expanded operand between more MFMAs, and their K loop is software-pipelined
-    // (expansions in the shadow of the MFMAs): per unit of work 3-12 % faster than the 128x128 shape, more the longer
-    // K is.  But a CU holds two such workgroups against four of the smaller shape, so what decides is the busiest
-    // CU: ceil(tiles / 256) tiles of either kind, the big ones twice the work each.  364 big tiles (two on some CUs)
-    // lose 5-12 % to 728 small ones (three), 392 (two) beat 784 (four) by 3-10 %, 784 lose again, 1456 win.  With K
-    // of 18 words only the types whose weights have two planes gained.  Which side gets four tiles: the dearer
-    // operand of TBN and BTN; TNN and, at long K, BNN measured 1-10 % faster with four filter tiles.
-    const long big_tiles = tiles(256, 128), small_tiles = tiles(128, 128);
-    const int unit_permille = a.G >= 72 ? 880 : (a.G >= 36 ? 920 : 970);  // time of a big tile / two small ones
-    // (packed output from the register-staged kernel, PC odd: its epilogue, a ballot per value, weighs more on eight
-    // tiles, and only many rounds of them pay)
-    const bool eight = a.qy != nullptr && a.PC % 2 != 0
-                           ? a.G >= 36 && big_tiles >= 2560
-                           : a.G >= (type == 0 || type == 2 ? 18 : 36) && big_tiles >= 160 &&
-                                 ((big_tiles + 255) / 256) * 2 * unit_permille < ((small_tiles + 255) / 256) * 1000;
-    if (eight) {
-        const bool wide = type == 1 || type == 0 || (type == 3 && a.G >= 72);
-        if (wide && a.KN >= 256) return 6;
-        if (a.KN >= 128) return 5;
+    const long kn64 = ((long)a.KN + 63) / 64 * 64;
+    // (packed output ranks the shapes as fp32 output does: the model's terms in Y also stand for what grows with M * KN)
+    const float y_mb = (float)a.M * (float)a.KN * 4e-6f;
+    int best = 2;
+    float best_cost = 0.f;
+    bool any = false;
+    for (int shape = 0; shape < kConvShapes; shape++) {
+        const int bm = kConvShapeTile[shape][0], bn = kConvShapeTile[shape][1], held = kConvShapeTile[shape][2];
+        if (bn >= 2 * kn64) continue;
+        if (shape == 3 && a.qy != nullptr) continue;  // the packed epilogues need tiles 64 filters wide
+        const long tiles = (long)((a.M + bm - 1) / bm) * ((a.KN + bn - 1) / bn);
+        const float n = (float)((tiles + 255) / 256), rounds = (float)(((tiles + 255) / 256 + held - 1) / held);
+        const float busy = tiles >= 256 ? 1.f : (float)tiles / 256.f;
+        const float f[kConvShapeFeatures] = {(float)a.G * n, (float)a.G * rounds, rounds, n, y_mb, y_mb * busy, busy, 1.f};
+        float cost = 0.f;
+        for (int i = 0; i < kConvShapeFeatures; i++) cost += kConvShapeCost[type][shape][i] * f[i];
+        if (!any || cost < best_cost) {
+            any = true;
+            best = shape;
+            best_cost = cost;
+        }
     }
-    if (a.KN > 64 && tiles(128, 128) >= (a.G >= 18 ? enough : (type == 3 ? 4096 : 1536))) return 0;
-    // one tile of filters: 256 rows per workgroup halve the expansions per MFMA of the 128x64 shape (two-plane
-    // operands gain 20 %, BNN 5-9 % on the largest launches only)
-    if (a.KN <= 64 && tiles(256, 64) >= (type != 3 ? 1024 : 4096)) return 4;
-    // a handful of words of K (1x1 layers on few channels): the 64x64 shape's short prologue wins
-    if (a.G <= 4 && tiles(64, 64) >= 192) return 2;
-    if (tiles(128, 64) >= enough) return 1;
-    if (tiles(64, 64) >= 192 || a.qy != nullptr) return 2;  // the packed epilogue needs tiles 64 filters wide
-    return 3;
+    return best;
 }
 
 hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream)

@@ -1,0 +1,125 @@
+"""Fits the cost model conv_mfma_shape() chooses the workgroup shape with and writes tab_amd/csrc/tab_conv_shape_model.h.
+
+Input: conv_shape_timings.txt (collect_conv_shape_timings.py): per (type, layer) the duration of every shape.
+Model, per (type, shape): duration ~ c . f with the features
+    f = [G*n, G*rounds, rounds, n, Y, Y*busy, busy, 1]
+    tiles  = ceil(M / BM) * ceil(KN / BN)            workgroups of the launch
+    n      = ceil(tiles / 256)                       tiles on the busiest of the 256 CUs
+    rounds = ceil(n / workgroups a CU holds)         how often that CU is refilled
+    busy   = min(1, tiles / 256)                     share of the CUs that have work at all
+    G      = KH*KW*PC words of K, Y = 4*M*KN bytes / 1e6
+fitted by least squares on relative error (ridge 1e-3; the N=16 set weighted threefold).  A shape whose filter tile is at least twice the (64-rounded)
+filter count is not a candidate.  The script prints the regret of the model's choice against the best measured shape:
+fitted on everything, and with each set held out in turn.
+
+    python tab_amd/tuning/fit_conv_shape_model.py        # needs numpy only"""
+import collections
+import os
+import re
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+SHAPES = {0: (128, 128, 4), 1: (128, 64, 4), 2: (64, 64, 4), 3: (32, 32, 8), 4: (256, 64, 3), 5: (256, 128, 2), 6: (128, 256, 2)}
+NFEAT = 8
+
+
+def parse(path):
+    rows, which = [], None
+    for line in open(path):
+        if line.startswith("##"):
+            which = line.split()[1]
+            continue
+        m = re.match(r"type (\d) N(\d+)_(\d+)x(\d+)x(\d+)->(\d+)_k(\d+)x(\d+)_p(\d)(\d)_s(\d)(\d)\s+\| (.*)", line)
+        if not m:
+            continue
+        t, N, H, W, C, KN, kh, kw, p1, p2, s1, s2 = map(int, m.groups()[:12])
+        OH, OW = (H + 2 * p1 - kh + 1) // s1, (W + 2 * p2 - kw + 1) // s2  # TAB_GEMM.cu:354-357
+        times = {int(a.split(":")[0]): float(a.split(":")[1]) for a in m.group(13).split()}
+        rows.append(dict(set=which, type=t, M=N * OH * OW, KN=KN, G=kh * kw * ((C + 63) // 64), times=times, name=line.split()[2]))
+    return rows
+
+
+def eligible(r, s):
+    return SHAPES[s][1] < 2 * (-(-r["KN"] // 64) * 64) and s in r["times"]
+
+
+def features(r, s):
+    BM, BN, held = SHAPES[s]
+    tiles = -(-r["M"] // BM) * -(-r["KN"] // BN)
+    n = -(-tiles // 256)
+    rounds = -(-n // held)
+    busy = min(1.0, tiles / 256.0)
+    Y = r["M"] * r["KN"] * 4e-6
+    return [r["G"] * n, r["G"] * rounds, rounds, n, Y, Y * busy, busy, 1.0]
+
+
+def fit(rows, ridge=1e-3):
+    coef = {}
+    for s in SHAPES:
+        for t in range(4):
+            X = np.array([features(r, s) for r in rows if r["type"] == t and eligible(r, s)])
+            y = np.array([r["times"][s] for r in rows if r["type"] == t and eligible(r, s)])
+            w = 1.0 / np.maximum(y, 1.0)  # relative error; the latency-bound N=16 set, the benchmark's headline, counts threefold
+            w = w * np.array([3.0 if r["set"] == "rn16" else 1.0 for r in rows if r["type"] == t and eligible(r, s)])
+            A, b = X * w[:, None], y * w
+            coef[(t, s)] = np.linalg.solve(A.T @ A + ridge * np.eye(NFEAT), A.T @ b)
+    return coef
+
+
+def choose(coef, r):
+    return min((s for s in SHAPES if eligible(r, s)), key=lambda s: (float(coef[(r["type"], s)] @ np.array(features(r, s))), s))
+
+
+def regret(rows, coef):
+    chosen = best = 0.0
+    per = collections.defaultdict(lambda: [0.0, 0.0])
+    for r in rows:
+        c, b = r["times"][choose(coef, r)], min(r["times"].values())
+        chosen += c
+        best += b
+        per[r["set"]][0] += c
+        per[r["set"]][1] += b
+    return chosen / best - 1, {k: v[0] / v[1] - 1 for k, v in per.items()}
+
+
+def main():
+    rows = parse(os.path.join(HERE, "conv_shape_timings.txt"))
+    coef = fit(rows)
+    total, per = regret(rows, coef)
+    sets = sorted(per)
+    held_chosen = held_best = 0.0
+    held = {}
+    for hold in sets:
+        c = fit([r for r in rows if r["set"] != hold])
+        g, _ = regret([r for r in rows if r["set"] == hold], c)
+        held[hold] = g
+        for r in rows:
+            if r["set"] == hold:
+                held_chosen += r["times"][choose(c, r)]
+                held_best += min(r["times"].values())
+    print(f"{len(rows)} cases; regret of the model's choice, fitted on all: {total:.2%} ({', '.join(f'{k} {v:.1%}' for k, v in sorted(per.items()))})")
+    print(f"each set held out of the fit in turn: {held_chosen / held_best - 1:.2%} ({', '.join(f'{k} {v:.1%}' for k, v in sorted(held.items()))})")
+    out = os.path.join(os.path.dirname(HERE), "csrc", "tab_conv_shape_model.h")
+    with open(out, "w") as f:
+        f.write("// Written by tab_amd/tuning/fit_conv_shape_model.py from tab_amd/tuning/conv_shape_timings.txt: do not edit.\n")
+        f.write("// Cost model of the matrix-core workgroup shapes: predicted duration (us) = kConvShapeCost[type][shape] . f,\n")
+        f.write("// f = {G*n, G*rounds, rounds, n, Y, Y*busy, busy, 1} (tiles on the busiest CU, refills of that CU, megabytes of Y,\n")
+        f.write("// share of the CUs with work).  Regret of the choice against the best measured shape over the\n")
+        f.write(f"// {len(rows)} fitted cases: {total:.2%}; with each layer set held out of the fit in turn: {held_chosen / held_best - 1:.2%}.\n")
+        f.write("#pragma once\n\nnamespace tab {\n\n")
+        f.write("constexpr int kConvShapes = 7, kConvShapeFeatures = 8;\n")
+        f.write("// rows x filters of the workgroup tile and workgroups a CU holds, per shape\n")
+        f.write("constexpr int kConvShapeTile[kConvShapes][3] = {" + ", ".join("{%d, %d, %d}" % SHAPES[s] for s in range(7)) + "};\n")
+        f.write("constexpr float kConvShapeCost[4][kConvShapes][kConvShapeFeatures] = {\n")
+        for t in range(4):
+            f.write("    {\n")
+            for s in range(7):
+                f.write("        {" + ", ".join("%.6gf" % v for v in coef[(t, s)]) + "},\n")
+            f.write("    },\n")
+        f.write("};\n\n}  // namespace tab\n")
+    print("wrote", out)
+
+
+if __name__ == "__main__":
+    main()
