@@ -638,12 +638,12 @@ def main():
         rn_ops, rn_ms, rn_pop_ms, rn_out_ms, rn_call_ms, rn_layers, rn_ok, rn_cpu_ms = 0, 0.0, 0.0, 0.0, 0.0, [], True, 0.0
         for i, l in enumerate(RESNET18_LAYERS):
             L = Layer(tab, torch, 3, 256, l, seed=i, on_device=True)
-            k_ms = graph_time_ms(torch, L.conv_kernel_only, 5, replays=4)
-            c_ms = graph_time_ms(torch, L.conv2d, 5, replays=4)
+            k_ms = graph_time_ms(torch, L.conv_kernel_only, 10, replays=4)
+            c_ms = graph_time_ms(torch, L.conv2d, 10, replays=4)
             tab.set_conv_kernel(tab.CONV_POPCOUNT, -1)
-            p_ms = graph_time_ms(torch, L.conv_kernel_only, 5, replays=4)
+            p_ms = graph_time_ms(torch, L.conv_kernel_only, 10, replays=4)
             tab.set_conv_kernel(tab.CONV_AUTO, -1)
-            o_ms = graph_time_ms(torch, L.conv_packed_out, 5, replays=4)
+            o_ms = graph_time_ms(torch, L.conv_packed_out, 10, replays=4)
             g = gate(oracle, L)
             cpu = cpu_reduced_batch(oracle, L)
             rn_ok = rn_ok and g["bit_exact_vs_cpu"]
@@ -683,10 +683,10 @@ def main():
         sweep = {}
         for type in range(4):
             L = Layer(tab, torch, type, 256, big, seed=7, relu=(type == 1), on_device=True)
-            k_ms = graph_time_ms(torch, L.conv_kernel_only, 5, replays=4)
+            k_ms = graph_time_ms(torch, L.conv_kernel_only, 10, replays=4)
             call_ms = graph_time_ms(torch, L.conv2d, 3, replays=3)
             tab.set_conv_kernel(tab.CONV_POPCOUNT, -1)
-            p_ms = graph_time_ms(torch, L.conv_kernel_only, 5, replays=4)
+            p_ms = graph_time_ms(torch, L.conv_kernel_only, 10, replays=4)
             tab.set_conv_kernel(tab.CONV_AUTO, -1)
             sweep[TYPE_NAMES[type]] = {"conv_kernel_ms": round(k_ms, 3), "call_ms": round(call_ms, 3),
                                        "conv_kernel_tops": round(L.ops / k_ms / 1e9, 1),
@@ -709,7 +709,7 @@ def main():
                 row = {}
                 for type in range(4):
                     L = Layer(tab, torch, type, n_batch, lay, seed=3, on_device=True)
-                    row[TYPE_NAMES[type]] = round(L.ops / graph_time_ms(torch, L.conv_kernel_only, 5, replays=3) / 1e9, 1)
+                    row[TYPE_NAMES[type]] = round(L.ops / graph_time_ms(torch, L.conv_kernel_only, 10, replays=3) / 1e9, 1)
                     more_ok = more_ok and gate(oracle, L)["bit_exact_vs_cpu"]
                     if type == 3:
                         row["cpu_BNN_tops_extrapolated"] = cpu_reduced_batch(oracle, L)["cpu_tops"]
