@@ -183,25 +183,38 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
         }
     };
     // Software pipeline over the MFMA steps (PIPELINED): while the matrix cores work on step s the vector unit expands
-    // the operands of step s + 1 into the other set of operand registers, one operand after each MFMA (a wave issues in
+    // the operands of step s + 1 into the other set of operand registers, a few dwords after each MFMA (a wave issues in
     // order: expansions written in front of their own MFMAs leave the matrix pipe idle meanwhile).  The raw words of a
     // pair are read from LDS a step before their first expansion; those of the next chunk's first pair right after the
     // barrier, which therefore stands before the chunk's last step.  The order is pinned with scheduling barriers: left
     // alone, the scheduler sinks the LDS reads to their first use and the wave waits for LDS in the middle of the MFMAs.
     i32x8 af[2][PIPELINED ? TM : 1], bf[2][PIPELINED ? TN : 1];
-    // operand e of a step, in the order the MFMAs need them: A0, B0 .. B(TN-1), A1 .. A(TM-1)
-    auto expand_one = [&](int e, int pair, int h, int set) {
+    // piece q of a step's expansions: dword q % 4 of operand q / 4, the operands in the order the MFMAs need them:
+    // A0, B0 .. B(TN-1), A1 .. A(TM-1).  (Indexing the whole expansion leaves the other three dwords to dead-code
+    // elimination.)  Dword-sized pieces spread the vector work evenly over the MFMAs: whole operands of a ternary side
+    // (12 instructions) outlast the MFMA they follow.
+    auto expand_piece = [&](int q, int pair, int h, int set) {
+        const int e = q / 4, d = q % 4;
         if (e == 0 || e > TN) {
             const int mt = e == 0 ? 0 : e - TN;
             const uint32_t *w = a_w[pair & 1][mt];
-            af[set][mt] = expand_operand<TYPE, 0>(w[h], w[2 * (APL - 1) + h], consts);
+            af[set][mt][d] = expand_operand<TYPE, 0>(w[h], w[2 * (APL - 1) + h], consts)[d];
         } else {
             const int nt = e - 1;
             const uint32_t *w = b_w[pair & 1][nt];
-            bf[set][nt] = expand_operand<TYPE, 1>(w[h], w[2 * (BPL - 1) + h], consts);
-            if (TYPE == 2) b_nonzero[nt] += __builtin_popcount(w[2 + h]);  // (the zeros past the last chunk add nothing)
+            bf[set][nt][d] = expand_operand<TYPE, 1>(w[h], w[2 * (BPL - 1) + h], consts)[d];
+            if (TYPE == 2 && d == 0) b_nonzero[nt] += __builtin_popcount(w[2 + h]);  // (the zeros past the last chunk add nothing)
         }
     };
+    if constexpr (PIPELINED) {
+#pragma unroll
+        for (int set = 0; set < 2; set++) {
+#pragma unroll
+            for (int mt = 0; mt < TM; mt++) af[set][mt] = i32x8{0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int nt = 0; nt < TN; nt++) bf[set][nt] = i32x8{0, 0, 0, 0, 0, 0, 0, 0};
+        }
+    }
 
     const int wave_m0 = m0 + wm * (32 * TM), wave_n0 = n0 + wn * (32 * TN);
 #pragma unroll
@@ -219,7 +232,7 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
     if constexpr (PIPELINED) {
         read_pair(lds, 0);
 #pragma unroll
-        for (int e = 0; e < NE; e++) expand_one(e, 0, 0, 0);
+        for (int q = 0; q < 4 * NE; q++) expand_piece(q, 0, 0, 0);
     }
 
     for (int chunk = 0; chunk < p.nchunks; chunk++) {
@@ -245,7 +258,7 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
                 __builtin_amdgcn_sched_barrier(0);
                 // the last step's expansions wait for the reads just issued: two MFMAs go first
                 const int delay = last ? 2 : 0;
-                const int per = (NE + (NM - delay) - 1) / (NM - delay);
+                const int per = (4 * NE + (NM - delay) - 1) / (NM - delay);  // pieces after each MFMA
                 const int npair = last ? 0 : (s + 1) / 2, nh = (s + 1) % 2;
                 int done = 0;
 #pragma unroll
@@ -254,10 +267,10 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
                     acc[mt][nt] = PACKED ? __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[s & 1][nt], af[s & 1][mt], acc[mt][nt], 4, 4, 0, 0, 0, 0)
                                          : __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[s & 1][mt], bf[s & 1][nt], acc[mt][nt], 4, 4, 0, 0, 0, 0);
                     __builtin_amdgcn_sched_barrier(0);
-                    const int upto = i < delay ? 0 : ((i + 1 - delay) * per < NE ? (i + 1 - delay) * per : NE);
+                    const int upto = i < delay ? 0 : ((i + 1 - delay) * per < 4 * NE ? (i + 1 - delay) * per : 4 * NE);
 #pragma unroll
-                    for (int e = 0; e < NE; e++)
-                        if (e >= done && e < upto) expand_one(e, npair, nh, (s + 1) & 1);
+                    for (int q = 0; q < 4 * NE; q++)
+                        if (q >= done && q < upto) expand_piece(q, npair, nh, (s + 1) & 1);
                     done = upto;
                     __builtin_amdgcn_sched_barrier(0);
                 }
