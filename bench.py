@@ -625,9 +625,15 @@ def main():
             # the same values read as NCHW (256x256x56x56): the quantizer of PyTorch-layout callers
             xn = xq.view(qN, qC, qH, qW)
             ms = event_time_ms(torch, lambda: tab.QuantizeNCHW(xn, ths, bitwidth, qN, qC, qH, qW), 20)
+            qn, btn_n = tab.QuantizeNCHW(xn, ths, bitwidth, qN, qC, qH, qW)
+            ok = True
+            for n in (0, qN // 2, qN - 1):  # whole images against the CPU quantizer's NCHW reading
+                q_o, b_o = oracle.quantize_nchw(xn[n:n + 1].cpu().numpy(), ths[n:n + 1].cpu().numpy(), bitwidth, 1, qC, qH, qW)
+                ok = ok and bool(np.array_equal(qn[n:n + 1].cpu().numpy(), q_o)) and int(btn_n[n]) == int(b_o[0])
             quant[f"nchw_bitwidth{bitwidth}"] = {"us": round(ms * 1e3, 1), "GBps": round(nbytes / ms / 1e6, 1),
-                                                 "frac_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
-            del qx
+                                                 "frac_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
+                                                 "bit_exact_vs_cpu": ok, "images_checked": 3}
+            del qx, qn
         ms = event_time_ms(torch, lambda: tab.Threshold(xq, qN, 0.7), 20)
         quant["threshold_abs_mean"] = {"us": round(ms * 1e3, 1), "GBps": round(4 * qN * qH * qW * qC / ms / 1e6, 1),
                                        "frac_hbm_peak": round(4 * qN * qH * qW * qC / ms / 1e6 / HBM_PEAK_GBS, 4)}
@@ -743,7 +749,7 @@ def main():
             result["cpu_baseline"]["gpu_bit_exact_vs_cpu"] and result["tnn_single_image_32x32x64"]["bit_exact_vs_cpu"]
             and all(t["bit_exact_vs_cpu"] for t in tern.values()) and rn_ok and more_ok and vgg_ok
             and all(v["bit_exact_vs_cpu"] for v in sweep.values())
-            and all(quant[f"bitwidth{b}"]["bit_exact_vs_cpu"] for b in (1, 2)))
+            and all(quant[f"{f}bitwidth{b}"]["bit_exact_vs_cpu"] for b in (1, 2) for f in ("", "nchw_")))
     print(json.dumps(result))
 
 
