@@ -54,6 +54,14 @@ EDGE_CASES = [
     (1, 12, 12, 640, 40, 3, 3, 1, 1, 2, 2),   # PC = 10
     (2, 8, 8, 384, 70, 1, 1, 0, 0, 1, 1),     # PC = 6, K = one tap
     (3, 6, 6, 768, 33, 3, 3, 1, 1, 1, 1),     # PC = 12, small launch: twelve-word chunks
+    (2, 5, 5, 64, 8, 3, 3, 3, 3, 1, 1),       # padding as wide as the kernel: the outer outputs see padding only
+    (2, 13, 13, 128, 8, 3, 3, 1, 1, 4, 4),    # stride beyond the kernel: pixels between the windows are never read
+    (3, 1, 17, 128, 12, 1, 3, 0, 1, 1, 1),    # images of one line
+    (2, 17, 1, 64, 12, 3, 1, 1, 0, 2, 1),     # images of one column
+    (1, 9, 9, 1, 3, 3, 3, 1, 1, 1, 1),        # one channel: 63 tail bits in every word
+    (2, 8, 12, 64, 9, 1, 7, 0, 3, 1, 1),      # 1x7 kernel
+    (40, 2, 2, 64, 5, 2, 2, 0, 0, 1, 1),      # one output pixel per image: a tile of rows spans 40 images
+    (3, 4, 4, 2048, 6, 2, 2, 1, 1, 1, 1),     # PC = 32
 ]
 
 

@@ -48,6 +48,10 @@ CASES = [
     (2, 10, 10, 192, 130, 3, 3, 1, 1, 1, 1),   # three words of filters, the last one 2 bits
     (5, 5, 5, 256, 96, 3, 3, 0, 0, 1, 1),      # 9 output pixels per image: a tile spans several images
     (2, 16, 16, 64, 200, 1, 1, 0, 0, 2, 2),    # 1x1 stride 2
+    (2, 5, 5, 64, 72, 3, 3, 3, 3, 1, 1),       # padding as wide as the kernel
+    (40, 2, 2, 128, 65, 2, 2, 0, 0, 1, 1),     # one output pixel per image: a tile of rows spans 40 images and thresholds
+    (3, 1, 17, 128, 33, 1, 3, 0, 1, 1, 1),     # images of one line
+    (2, 13, 13, 256, 129, 3, 3, 1, 1, 4, 4),   # stride beyond the kernel
 ]
 
 
