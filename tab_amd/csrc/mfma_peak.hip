@@ -4,9 +4,9 @@
 // per-tile expansion work of each conv type in front of it, for the tiles per wave and workgroups per CU the conv
 // kernel runs (2x2 at up to four workgroups, 4x2 / 2x4 at two), (3) measures how many independent vector
 // instructions fit in an MFMA's shadow, (4) compares the two orders of a step of the conv kernel's loop: all
-// expansions, then the MFMAs (serial), against the next step's expansions one after each MFMA of this step
-// into a second set of operand registers (pipelined), with the expansion constants in registers as in the
-// kernel, and reports the shader clock each run held (s_memtime over s_memrealtime).
+// expansions, then the MFMAs (serial), against the next step's expansions spread dword by dword over the MFMAs of
+// this step, into a second set of operand registers (pipelined), with the expansion constants in registers as in
+// the kernel, and reports the shader clock each run held (s_memtime over s_memrealtime).
 // Register-resident: no memory traffic in the timed loops.
 #include <hip/hip_runtime.h>
 #include <cstdio>
@@ -20,7 +20,8 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 #define M2 0x44444444u
 #define M3 0x88888888u
 // E2M1 nibble: bit3 sign, bits 2:1 exponent, bit0 mantissa: 0001=0.5 0010=1 0100=2
-// A-side weights per nibble bit j: (0.5, 1, 2, 2); B-side: (2, 1, 0.5, 0.5)
+// BNN: A-side weights per nibble bit j: (0.5, 1, 2, 2); B-side: (2, 1, 0.5, 0.5).  A ternary operand is +-2 or 0 in
+// every position, its binary partner +-0.5; two ternary operands give four times the sum.
 __device__ __forceinline__ v8i bin_a(uint32_t w)   // value (bit ? -1 : +1) * weight
 {
     v8i r = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -33,18 +34,19 @@ __device__ __forceinline__ v8i bin_b(uint32_t w)
     r[0] = (int)(((w << 3) & M3) | M2); r[1] = (int)(((w << 2) & M3) | M1); r[2] = (int)(((w << 1) & M3) | M0); r[3] = (int)((w & M3) | M0);
     return r;
 }
-__device__ __forceinline__ v8i ter_a(uint32_t s, uint32_t z)   // nz * (sign ? -1 : +1) * weight
+__device__ __forceinline__ v8i bin_half(uint32_t w)   // (bit ? -1 : +1) * 0.5
 {
     v8i r = {0, 0, 0, 0, 0, 0, 0, 0};
-    r[0] = (int)((z & M0) | ((s << 3) & M3)); r[1] = (int)((z & M1) | ((s << 2) & M3));
-    r[2] = (int)((z & M2) | ((s << 1) & M3)); r[3] = (int)(((z >> 1) & M2) | (s & M3));
+    r[0] = (int)(((w << 3) & M3) | M0); r[1] = (int)(((w << 2) & M3) | M0); r[2] = (int)(((w << 1) & M3) | M0); r[3] = (int)((w & M3) | M0);
     return r;
 }
-__device__ __forceinline__ v8i ter_b(uint32_t s, uint32_t z)
+// nz * (sign ? -2 : +2): pair words of the even and of the odd positions, (nonzero, sign) adjacent, then the pairs
+// as the top two bits of each nibble
+__device__ __forceinline__ v8i ter(uint32_t s, uint32_t z)
 {
     v8i r = {0, 0, 0, 0, 0, 0, 0, 0};
-    r[0] = (int)(((z << 2) & M2) | ((s << 3) & M3)); r[1] = (int)((z & M1) | ((s << 2) & M3));
-    r[2] = (int)(((z >> 2) & M0) | ((s << 1) & M3)); r[3] = (int)(((z >> 3) & M0) | (s & M3));
+    const uint32_t a = (z & 0x55555555u) | ((s << 1) & 0xAAAAAAAAu), b = (s & 0xAAAAAAAAu) | ((z >> 1) & 0x55555555u);
+    r[0] = (int)((a << 2) & 0xCCCCCCCCu); r[1] = (int)((b << 2) & 0xCCCCCCCCu); r[2] = (int)(a & 0xCCCCCCCCu); r[3] = (int)(b & 0xCCCCCCCCu);
     return r;
 }
 __device__ __forceinline__ v16f mfma(v8i a, v8i b, v16f c) { return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 4, 4, 0, 0, 0, 0); }
@@ -52,12 +54,67 @@ __device__ __forceinline__ v16f mfma(v8i a, v8i b, v16f c) { return __builtin_am
 __global__ void k_check(const uint32_t *As, const uint32_t *Az, const uint32_t *Bs, const uint32_t *Bz, float *C, int mode)
 {
     const int lane = threadIdx.x, r = lane & 31, kb = lane >> 5;
-    v8i a = (mode & 1) ? ter_a(As[r * 2 + kb], Az[r * 2 + kb]) : bin_a(As[r * 2 + kb]);
-    v8i b = (mode & 2) ? ter_b(Bs[r * 2 + kb], Bz[r * 2 + kb]) : bin_b(Bs[r * 2 + kb]);
+    v8i a = (mode & 1) ? ter(As[r * 2 + kb], Az[r * 2 + kb]) : (mode & 2) ? bin_half(As[r * 2 + kb]) : bin_a(As[r * 2 + kb]);
+    v8i b = (mode & 2) ? ter(Bs[r * 2 + kb], Bz[r * 2 + kb]) : (mode & 1) ? bin_half(Bs[r * 2 + kb]) : bin_b(Bs[r * 2 + kb]);
     v16f c = {0};
     c = mfma(a, b, c);
     for (int j = 0; j < 4; j++)
         for (int i = 0; i < 4; i++) C[(8 * j + 4 * kb + i) * 32 + r] = c[4 * j + i];
+}
+// The conv kernel's expansions with their constants in registers (masks in SGPRs, patterns in VGPRs): 7 vector
+// instructions for a binary operand, 10 for a ternary one (a shift and a three-input bit operation per pair word, a
+// shift and an AND for dwords 0 and 1, an AND for dwords 2 and 3), dword by dword.
+struct ExpandRegs { uint32_t m3, p0, p1, p2, even, odd, pair; };
+__device__ __forceinline__ ExpandRegs expand_regs()
+{
+    ExpandRegs k = {M3, M0, M1, M2, 0x55555555u, 0xAAAAAAAAu, 0xCCCCCCCCu};
+    asm volatile("" : "+s"(k.m3), "+s"(k.even), "+s"(k.odd), "+s"(k.pair));
+    asm volatile("" : "+v"(k.p0), "+v"(k.p1), "+v"(k.p2));
+    return k;
+}
+__device__ __forceinline__ int bin_dword(uint32_t w, int d, const ExpandRegs &k)
+{
+    return (int)(((w << (3 - d)) & k.m3) | (d == 0 ? k.p0 : d == 1 ? k.p1 : k.p2));
+}
+__device__ __forceinline__ int ter_dword(uint32_t s, uint32_t z, int d, uint32_t (&pw)[2], const ExpandRegs &k)
+{
+    if (d == 0) {
+        const uint32_t s1 = s << 1;
+        uint32_t a = ((z ^ s1) & k.even) ^ s1;
+        asm("" : "+v"(a));  // opaque, or the optimiser re-derives every dword from s and z
+        pw[0] = a;
+        return (int)((a << 2) & k.pair);
+    }
+    if (d == 1) {
+        const uint32_t z1 = z >> 1;
+        uint32_t b = ((s ^ z1) & k.odd) ^ z1;
+        asm("" : "+v"(b));
+        pw[1] = b;
+        return (int)((b << 2) & k.pair);
+    }
+    return (int)(pw[d - 2] & k.pair);
+}
+__device__ __forceinline__ v8i ter_op(uint32_t s, uint32_t z, const ExpandRegs &k)
+{
+    v8i r = {0, 0, 0, 0, 0, 0, 0, 0};
+    uint32_t pw[2];
+#pragma unroll
+    for (int d = 0; d < 4; d++) r[d] = ter_dword(s, z, d, pw, k);
+    return r;
+}
+__device__ __forceinline__ v8i bin_op(uint32_t w, const ExpandRegs &k)
+{
+    v8i r = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int d = 0; d < 4; d++) r[d] = bin_dword(w, d, k);
+    return r;
+}
+__device__ __forceinline__ v8i half_op(uint32_t w, const ExpandRegs &k)
+{
+    v8i r = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int d = 0; d < 4; d++) r[d] = (int)(((w << (3 - d)) & k.m3) | k.p0);
+    return r;
 }
 // MODE 0: mfma only; 1: BNN expansions; 2: TNN expansions; 3: TBN.  TM x TN MFMA tiles per wave, one expansion per
 // operand tile and step as in the conv kernel: 2x2 (the 128x128 workgroup tile), 4x2 and 2x4 (256x128 / 128x256).
@@ -68,13 +125,14 @@ __global__ __launch_bounds__(256) void k_tput(float *out, int iters, uint32_t se
     for (int i = 0; i < TM; i++) for (int j = 0; j < TN; j++) for (int e = 0; e < 16; e++) c[i][j][e] = 0;
     uint32_t w[2 * (TM + TN)];
     for (int i = 0; i < 2 * (TM + TN); i++) w[i] = seed * (threadIdx.x + 1) * (2 * i + 1);
+    const ExpandRegs k = expand_regs();
     v8i a[TM], b[TN];
     for (int i = 0; i < TM; i++) a[i] = bin_a(w[i]);
     for (int i = 0; i < TN; i++) b[i] = bin_b(w[TM + i]);
     for (int it = 0; it < iters; it++) {
         if (MODE != 0) {
-            for (int i = 0; i < TM; i++) a[i] = (MODE == 1) ? bin_a(w[i]) : ter_a(w[i], w[TM + TN + i]);
-            for (int i = 0; i < TN; i++) b[i] = (MODE == 2) ? ter_b(w[TM + i], w[2 * TM + TN + i]) : bin_b(w[TM + i]);
+            for (int i = 0; i < TM; i++) a[i] = (MODE == 1) ? bin_op(w[i], k) : ter_op(w[i], w[TM + TN + i], k);
+            for (int i = 0; i < TN; i++) b[i] = (MODE == 2) ? ter_op(w[TM + i], w[2 * TM + TN + i], k) : (MODE == 3) ? half_op(w[TM + i], k) : bin_op(w[TM + i], k);
             w[0] += 0x9e3779b9u; for (int i = 1; i < 2 * (TM + TN); i++) w[i] ^= w[i - 1];
         }
 #pragma unroll
@@ -139,49 +197,35 @@ template <int NV> int shadow(int bpc)
     return 0;
 }
 
-// The conv kernel's expansions with their constants in registers (mask in an SGPR, patterns in VGPRs): 7 vector
-// instructions for a binary operand, 12 for a ternary one.
-struct ExpandRegs { uint32_t m3, p0, p1, p2, m0, m1, m2; };
-__device__ __forceinline__ ExpandRegs expand_regs()
-{
-    ExpandRegs k = {M3, M0, M1, M2, M0, M1, M2};
-    asm volatile("" : "+s"(k.m3), "+s"(k.m0), "+s"(k.m1), "+s"(k.m2));
-    asm volatile("" : "+v"(k.p0), "+v"(k.p1), "+v"(k.p2));
-    return k;
-}
-__device__ __forceinline__ v8i bin_regs(uint32_t w, const ExpandRegs &k)
-{
-    v8i r = {0, 0, 0, 0, 0, 0, 0, 0};
-    r[0] = (int)(((w << 3) & k.m3) | k.p0); r[1] = (int)(((w << 2) & k.m3) | k.p1); r[2] = (int)(((w << 1) & k.m3) | k.p2); r[3] = (int)((w & k.m3) | k.p2);
-    return r;
-}
-__device__ __forceinline__ v8i ter_regs(uint32_t s, uint32_t z, const ExpandRegs &k)
-{
-    v8i r = {0, 0, 0, 0, 0, 0, 0, 0};
-    r[0] = (int)((z & k.m0) | ((s << 3) & k.m3)); r[1] = (int)((z & k.m1) | ((s << 2) & k.m3));
-    r[2] = (int)((z & k.m2) | ((s << 1) & k.m3)); r[3] = (int)(((z >> 1) & k.m2) | (s & k.m3));
-    return r;
-}
 // TER: ternary operands on both sides.  PIPE 0: the TM + TN expansions of a step, then its TM * TN MFMAs; 1: the
-// MFMAs of a step with the next step's expansions one after each, into the other operand set.  Order pinned.
+// MFMAs of a step with the next step's expansions spread over them dword by dword, into the other operand set.
+// Order pinned.
 template <int TER, int PIPE, int TM, int TN>
 __global__ __launch_bounds__(256) void k_step_order(float *out, long long *clocks, int iters, uint32_t seed)
 {
     constexpr int NE = TM + TN, NM = TM * TN;
+    constexpr int PER = (4 * NE + NM - 1) / NM;  // dwords after each MFMA
     v16f c[TM][TN];
     for (int i = 0; i < TM; i++) for (int j = 0; j < TN; j++) for (int e = 0; e < 16; e++) c[i][j][e] = 0;
     uint32_t w[2 * NE];
     for (int i = 0; i < 2 * NE; i++) w[i] = seed * (threadIdx.x + 1) * (2 * i + 1);
     const ExpandRegs k = expand_regs();
     v8i op[2][NE];
-    for (int e = 0; e < NE; e++) op[0][e] = op[1][e] = bin_regs(w[e], k);
+    uint32_t pw[2];
+    auto piece = [&](int q, int set) {
+        const int e = q / 4, d = q % 4;
+        op[set][e][d] = TER ? ter_dword(w[e], w[NE + e], d, pw, k) : bin_dword(w[e], d, k);
+    };
+    for (int set = 0; set < 2; set++) for (int e = 0; e < NE; e++) op[set][e] = v8i{0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int q = 0; q < 4 * NE; q++) piece(q, 0);
     const long long t0 = clock64(), r0 = wall_clock64();
     for (int it = 0; it < iters; it++) {
 #pragma unroll
         for (int s = 0; s < 2; s++) {
             if (PIPE == 0) {
 #pragma unroll
-                for (int e = 0; e < NE; e++) op[s][e] = TER ? ter_regs(w[e], w[NE + e], k) : bin_regs(w[e], k);
+                for (int q = 0; q < 4 * NE; q++) piece(q, s);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int i = 0; i < NM; i++) c[i / TN][i % TN] = mfma(op[s][i / TN], op[s][TM + i % TN], c[i / TN][i % TN]);
@@ -191,7 +235,9 @@ __global__ __launch_bounds__(256) void k_step_order(float *out, long long *clock
                 for (int i = 0; i < NM; i++) {
                     c[i / TN][i % TN] = mfma(op[s][i / TN], op[s][TM + i % TN], c[i / TN][i % TN]);
                     __builtin_amdgcn_sched_barrier(0);
-                    if (i < NE) op[s ^ 1][i] = TER ? ter_regs(w[i], w[NE + i], k) : bin_regs(w[i], k);
+#pragma unroll
+                    for (int q = i * PER; q < (i + 1) * PER; q++)
+                        if (q < 4 * NE) piece(q, s ^ 1);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
@@ -245,7 +291,7 @@ int main()
                 const int bv = (mode & 2) ? val_t(h[2][n * 2 + q], h[3][n * 2 + q], kk) : val_b(h[2][n * 2 + q], kk);
                 s += av * bv;
             }
-            bad += hC[m * 32 + n] != (float)s;
+            bad += hC[m * 32 + n] != (float)(mode == 3 ? 4 * s : s);  // ternary x ternary: +-2 x +-2
         }
         printf("check A %s x B %s: %d mismatches of 1024 (C[0][0]=%g)\n", (mode & 1) ? "ternary" : "binary", (mode & 2) ? "ternary" : "binary", bad, hC[0]);
     }

@@ -45,14 +45,18 @@ constexpr uint32_t kBit0 = 0x11111111u, kBit1 = 0x22222222u, kBit2 = 0x44444444u
 struct ExpandConsts {
     uint32_t sign_bits;          // kBit3, SGPR
     uint32_t half, one, two;     // the E2M1 patterns of 0.5, 1, 2 in every nibble, VGPRs
-    __device__ __forceinline__ ExpandConsts() : sign_bits(kBit3), half(kBit0), one(kBit1), two(kBit2)
+    uint32_t even, odd, pair;    // masks of the ternary expansion, SGPRs
+    __device__ __forceinline__ ExpandConsts()
+        : sign_bits(kBit3), half(kBit0), one(kBit1), two(kBit2), even(0x55555555u), odd(0xAAAAAAAAu), pair(0xCCCCCCCCu)
     {
         asm volatile("" : "+s"(sign_bits));
         asm volatile("" : "+v"(half), "+v"(one), "+v"(two));
+        asm("" : "+s"(even), "+s"(odd), "+s"(pair));
     }
 };
 
-// SIDE 0 = activation (weights 0.5, 1, 2, 2), SIDE 1 = weight operand (2, 1, 0.5, 0.5)
+// Binary operand of BNN.  SIDE 0 = activation (weights 0.5, 1, 2, 2), SIDE 1 = weight operand (2, 1, 0.5, 0.5): the
+// products are +-1 and both sides have the same number of instructions.
 template <int SIDE>
 __device__ __forceinline__ i32x8 expand_binary(uint32_t w, const ExpandConsts &c)
 {
@@ -65,22 +69,58 @@ __device__ __forceinline__ i32x8 expand_binary(uint32_t w, const ExpandConsts &c
     return r;
 }
 
-template <int SIDE>
+// Dword d of the binary partner of a ternary operand (TBN weights, BTN activations): +-0.5 in every dword.
+__device__ __forceinline__ int half_binary_dword(uint32_t w, int d, const ExpandConsts &c)
+{
+    return (int)(((w << (3 - d)) & c.sign_bits) | c.half);
+}
+
+// Ternary operand (either side), 10 vector instructions: the (nonzero, sign) bits of the even positions of a slice are
+// merged into one word of adjacent pairs and those of the odd positions into another (a shift and one three-input
+// v_bitop3_b32 each); a pair is already the two top bits of an E2M1 nibble, sign and the exponent bit of 2, so dwords 2
+// and 3 are one AND of a pair word and dwords 0 and 1 a shift and an AND.  Dword d holds the elements 4i + d of the
+// slice, as in the binary expansions.  Every ternary element is +-2 or (+-)0; a binary partner is +-0.5 throughout
+// (products +-1), and two ternary sides give four times the sum, which the kernels scale back with scale_ternary_sums
+// (exact: 4 * 64 * G < 2^24 for every G the library takes).  With separate sign and magnitude masks per dword
+// ((s << k) & sign | (z >> j) & bit) the same operand took 12 instructions (activation side) or 14 (weight side).
+// d = 0 and d = 1 make the pair words and leave them in pw for d = 2 and d = 3.
+__device__ __forceinline__ int ternary_dword(uint32_t s, uint32_t z, int d, uint32_t (&pw)[2], const ExpandConsts &c)
+{
+    if (d == 0) {
+        const uint32_t s1 = s << 1;
+        uint32_t a = ((z ^ s1) & c.even) ^ s1;  // bit 2j = z[2j], bit 2j+1 = s[2j]
+        asm("" : "+v"(a));  // opaque: the optimiser otherwise re-derives each dword from s and z (14 instructions)
+        pw[0] = a;
+        return (int)((a << 2) & c.pair);
+    }
+    if (d == 1) {
+        const uint32_t z1 = z >> 1;
+        uint32_t b = ((s ^ z1) & c.odd) ^ z1;  // bit 2j = z[2j+1], bit 2j+1 = s[2j+1]
+        asm("" : "+v"(b));
+        pw[1] = b;
+        return (int)((b << 2) & c.pair);
+    }
+    return (int)(pw[d - 2] & c.pair);
+}
+
 __device__ __forceinline__ i32x8 expand_ternary(uint32_t s, uint32_t z, const ExpandConsts &c)
 {
     i32x8 r = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (SIDE == 0) {
-        r[0] = (int)(((s << 3) & c.sign_bits) | (z & kBit0));
-        r[1] = (int)(((s << 2) & c.sign_bits) | (z & kBit1));
-        r[2] = (int)(((s << 1) & c.sign_bits) | (z & kBit2));
-        r[3] = (int)((s & c.sign_bits) | ((z >> 1) & kBit2));
-    } else {
-        r[0] = (int)(((s << 3) & c.sign_bits) | ((z << 2) & kBit2));
-        r[1] = (int)(((s << 2) & c.sign_bits) | (z & kBit1));
-        r[2] = (int)(((s << 1) & c.sign_bits) | ((z >> 2) & kBit0));
-        r[3] = (int)((s & c.sign_bits) | ((z >> 3) & kBit0));
-    }
+    uint32_t pw[2];
+#pragma unroll
+    for (int d = 0; d < 4; d++) r[d] = ternary_dword(s, z, d, pw, c);
     return r;
+}
+
+// TNN: both operands are +-2, the accumulators hold four times the sums
+template <int TYPE, int TM, int TN>
+__device__ __forceinline__ void scale_ternary_sums(f32x16 (&acc)[TM][TN])
+{
+    if (TYPE != 0) return;
+#pragma unroll
+    for (int mt = 0; mt < TM; mt++)
+#pragma unroll
+        for (int nt = 0; nt < TN; nt++) acc[mt][nt] *= 0.25f;
 }
 
 // Type 4 (TAB_CPU.cpp:332-358): planes (hi, lo) of a level 0..3 on both sides; E2M1 holds 1 = 0010,
@@ -120,7 +160,12 @@ __device__ __forceinline__ i32x8 expand_operand(uint32_t p0, uint32_t p1, const 
     if (TYPE == 4) return expand_levels(p0, p1);
     if (TYPE == 5) return expand_fields(p0, p1);
     constexpr int PL = SIDE ? Planes<TYPE>::B : Planes<TYPE>::A;
-    return PL == 2 ? expand_ternary<SIDE>(p0, p1, c) : expand_binary<SIDE>(p0, c);
+    if (PL == 2) return expand_ternary(p0, p1, c);
+    if (TYPE == 3) return expand_binary<SIDE>(p0, c);
+    i32x8 r = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int d = 0; d < 4; d++) r[d] = half_binary_dword(p0, d, c);
+    return r;
 }
 
 // Epilogue shared by the matrix-core kernels: accumulator element 4*j + i of lane (kb, r) is
@@ -547,6 +592,7 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
         __syncthreads();
     }
 
+    scale_ternary_sums<TYPE>(acc);
     conv_mfma_epilogue<TYPE, TM, TN, KCH, KS>(p, acc, b_nonzero, wave_m0, wave_n0, lane, ks, partial);
 }
 

@@ -192,17 +192,26 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
     // piece q of a step's expansions: dword q % 4 of operand q / 4, the operands in the order the MFMAs need them:
     // A0, B0 .. B(TN-1), A1 .. A(TM-1).  (Indexing the whole expansion leaves the other three dwords to dead-code
     // elimination.)  Dword-sized pieces spread the vector work evenly over the MFMAs: whole operands of a ternary side
-    // (12 instructions) outlast the MFMA they follow.
+    // (10 instructions) outlast the MFMA they follow.
+    // (the ternary expansion goes dword by dword with its pair words kept in between: indexing the whole expansion
+    // would compute them once per piece)
+    uint32_t pair_words[2];
     auto expand_piece = [&](int q, int pair, int h, int set) {
         const int e = q / 4, d = q % 4;
         if (e == 0 || e > TN) {
             const int mt = e == 0 ? 0 : e - TN;
             const uint32_t *w = a_w[pair & 1][mt];
-            af[set][mt][d] = expand_operand<TYPE, 0>(w[h], w[2 * (APL - 1) + h], consts)[d];
+            if constexpr (TYPE <= 2)
+                af[set][mt][d] = APL == 2 ? ternary_dword(w[h], w[2 + h], d, pair_words, consts) : half_binary_dword(w[h], d, consts);
+            else
+                af[set][mt][d] = expand_operand<TYPE, 0>(w[h], w[2 * (APL - 1) + h], consts)[d];
         } else {
             const int nt = e - 1;
             const uint32_t *w = b_w[pair & 1][nt];
-            bf[set][nt][d] = expand_operand<TYPE, 1>(w[h], w[2 * (BPL - 1) + h], consts)[d];
+            if constexpr (TYPE <= 2)
+                bf[set][nt][d] = BPL == 2 ? ternary_dword(w[h], w[2 + h], d, pair_words, consts) : half_binary_dword(w[h], d, consts);
+            else
+                bf[set][nt][d] = expand_operand<TYPE, 1>(w[h], w[2 * (BPL - 1) + h], consts)[d];
             if (TYPE == 2 && d == 0) b_nonzero[nt] += __builtin_popcount(w[2 + h]);  // (the zeros past the last chunk add nothing)
         }
     };
@@ -313,6 +322,7 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
         }
     }
 
+    scale_ternary_sums<TYPE>(acc);
     if constexpr (PACKED) {
         // BTN hands its biases round through LDS: not before every wave has read its last operands (the pipelined
         // loop reads the zeros past the last chunk after the chunk's barrier and counts their nonzero weights)

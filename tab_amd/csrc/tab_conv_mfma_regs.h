@@ -227,6 +227,10 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(2,
                                : __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af, wf, acc[nt], 4, 4, 0, 0, 0, 0);
             }
         }
+        if (TYPE == 0) {  // both operands are +-2: four times the sums
+#pragma unroll
+            for (int nt = 0; nt < TN; nt++) acc[nt] *= 0.25f;
+        }
         // Every store goes through a buffer descriptor that ends with the tile's last live row, so pixels past M
         // (and, by an offset select, filters past KN) are dropped by the range check instead of branched round: with
         // no branch in the loop every iteration issues the same number of memory operations, and the wait for the

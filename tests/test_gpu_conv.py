@@ -315,3 +315,24 @@ def test_conv_rejects_wrong_sizes():
     qw4 = torch.zeros((4, 3, 3, 4, 1), dtype=torch.int64, device="cuda")
     with pytest.raises(RuntimeError, match="empty output"):
         tab_amd.Conv2d(x, qw4, ths, btn, 3, 0, 0, 1, 1, 1, 2, 2, 64 * 4, 4, 3, 3)
+
+
+@pytest.mark.parametrize("type", [0, 1, 2, 3])
+def test_longest_k_with_every_product_of_one_sign(type):
+    """K = 65535 words, the most the library takes, and filters whose products are all +1, all -1, or cancel: the
+    sums +-4194240 must come out exact (two ternary operands multiply as +-2 x +-2 and are scaled back, so their
+    accumulators reach 16776960, just below 2^24)."""
+    C, KN = 64 * 65535, 3
+    print(f"[case] Conv2d {TYPE_NAMES[type]} 1x1x{C}->{KN}", flush=True)
+    x = np.full((1, 1, 1, C), 1.0, dtype=np.float32)
+    w = np.ones((KN, 1, 1, C), dtype=np.float32)
+    w[1] = -1.0
+    w[2, :, :, 1::2] = -1.0
+    ths = np.array([0.5 if act_bits(type) == 2 else 0.0], dtype=np.float32)
+    w_ths = np.full(KN, 0.5 if weight_bits(type) == 2 else 0.0, dtype=np.float32)
+    qw, btn = oracle.quantize(w, w_ths, weight_bits(type), KN, 1, 1, C)
+    want = oracle.conv2d(x, qw, ths, btn, type, 0, 0, 1, 1, 1, 1, 1, C, KN, 1, 1)
+    assert want.reshape(-1).tolist() == [float(C), -float(C), 0.0]
+    y = tab_amd.Conv2d(torch.from_numpy(x).cuda(), torch.from_numpy(qw).cuda(), torch.from_numpy(ths).cuda(),
+                       torch.from_numpy(btn).cuda(), type, 0, 0, 1, 1, 1, 1, 1, C, KN, 1, 1)
+    assert np.array_equal(y.cpu().numpy(), want)
