@@ -365,10 +365,11 @@ hipError_t launch_conv_mfma(int type, const ConvArgs &args, int shape, hipStream
 // the measured duration of every shape on 280 (type, layer) cases (tab_conv_shape_model.h: the ResNet-18 layers at
 // N = 16 / 64 / 256, the VGG stack, the 28x28 sweep and layers of other geometries).  What the model's features say:
 // the busiest of the 256 CUs decides (ceil(tiles / 256) tiles of a shape land on it, and it is refilled when it holds
-// no more), K scales the loop, the size of Y the epilogue, and a launch smaller than the chip is as long as one tile.
+// no more), K scales the loop, the size of Y the epilogue (with a price of its own where K is at most nine words and
+// the launch is little but epilogue), and a launch smaller than the chip is as long as one tile.
 // A shape whose filter tile is at least twice the 64-rounded filter count is no candidate.  Regret of the choice
-// against the best measured shape: 1.5 % over the fitted cases, 2.3 % with each layer set held out of the fit in turn
-// (the thresholds this replaces: 2.8 % on the same measurements, 5.5 % on the geometries they were not made from).
+// against the best measured shape: 1.0 % over the fitted cases, 1.4 % with each layer set held out of the fit in turn
+// (the thresholds this replaces: 2.8 % on their measurements, 5.5 % on the geometries they were not made from).
 int conv_mfma_shape(int conv_type, const ConvArgs &a)
 {
     // the CPU-only types follow the type with the same planes: 4 like TNN, 5 like BNN
@@ -391,7 +392,8 @@ int conv_mfma_shape(int conv_type, const ConvArgs &a)
         const long tiles = (long)((a.M + bm - 1) / bm) * ((a.KN + bn - 1) / bn);
         const float n = (float)((tiles + 255) / 256), rounds = (float)(((tiles + 255) / 256 + held - 1) / held);
         const float busy = tiles >= 256 ? 1.f : (float)tiles / 256.f;
-        const float f[kConvShapeFeatures] = {(float)a.G * n, (float)a.G * rounds, rounds, n, y_mb, y_mb * busy, busy, 1.f};
+        const float f[kConvShapeFeatures] = {(float)a.G * n, (float)a.G * rounds, rounds, n, y_mb, y_mb * busy, busy, 1.f,
+                                             a.G <= 9 ? y_mb : 0.f};
         float cost = 0.f;
         for (int i = 0; i < kConvShapeFeatures; i++) cost += kConvShapeCost[type][shape][i] * f[i];
         if (!any || cost < best_cost) {

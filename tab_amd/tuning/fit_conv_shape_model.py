@@ -2,13 +2,14 @@
 
 Input: conv_shape_timings.txt (collect_conv_shape_timings.py): per (type, layer) the duration of every shape.
 Model, per (type, shape): duration ~ c . f with the features
-    f = [G*n, G*rounds, rounds, n, Y, Y*busy, busy, 1]
+    f = [G*n, G*rounds, rounds, n, Y, Y*busy, busy, 1, Y*[G <= 9]]
     tiles  = ceil(M / BM) * ceil(KN / BN)            workgroups of the launch
     n      = ceil(tiles / 256)                       tiles on the busiest of the 256 CUs
     rounds = ceil(n / workgroups a CU holds)         how often that CU is refilled
     busy   = min(1, tiles / 256)                     share of the CUs that have work at all
-    G      = KH*KW*PC words of K, Y = 4*M*KN bytes / 1e6
-fitted by least squares on relative error (ridge 1e-3; the N=16 set weighted threefold).  A shape whose filter tile is at least twice the (64-rounded)
+    G      = KH*KW*PC words of K, Y = 4*M*KN bytes / 1e6; the last feature gives the layers whose loop is a handful of
+             MFMAs (C = 64 with 3x3, 1x1) their own price per byte of Y: their launches are the epilogue
+fitted by least squares on relative error (ridge 1e-2; the N=16 set weighted threefold).  A shape whose filter tile is at least twice the (64-rounded)
 filter count is not a candidate.  The script prints the regret of the model's choice against the best measured shape:
 fitted on everything, and with each set held out in turn.
 
@@ -21,7 +22,7 @@ import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SHAPES = {0: (128, 128, 4), 1: (128, 64, 4), 2: (64, 64, 4), 3: (32, 32, 8), 4: (256, 64, 3), 5: (256, 128, 2), 6: (128, 256, 2)}
-NFEAT = 8
+NFEAT = 9
 
 
 def parse(path):
@@ -51,10 +52,10 @@ def features(r, s):
     rounds = -(-n // held)
     busy = min(1.0, tiles / 256.0)
     Y = r["M"] * r["KN"] * 4e-6
-    return [r["G"] * n, r["G"] * rounds, rounds, n, Y, Y * busy, busy, 1.0]
+    return [r["G"] * n, r["G"] * rounds, rounds, n, Y, Y * busy, busy, 1.0, Y if r["G"] <= 9 else 0.0]
 
 
-def fit(rows, ridge=1e-3):
+def fit(rows, ridge=1e-2):
     coef = {}
     for s in SHAPES:
         for t in range(4):
@@ -104,11 +105,11 @@ def main():
     with open(out, "w") as f:
         f.write("// Written by tab_amd/tuning/fit_conv_shape_model.py from tab_amd/tuning/conv_shape_timings.txt: do not edit.\n")
         f.write("// Cost model of the matrix-core workgroup shapes: predicted duration (us) = kConvShapeCost[type][shape] . f,\n")
-        f.write("// f = {G*n, G*rounds, rounds, n, Y, Y*busy, busy, 1} (tiles on the busiest CU, refills of that CU, megabytes of Y,\n")
-        f.write("// share of the CUs with work).  Regret of the choice against the best measured shape over the\n")
+        f.write("// f = {G*n, G*rounds, rounds, n, Y, Y*busy, busy, 1, Y*[G <= 9]} (tiles on the busiest CU, refills of that CU, megabytes\n")
+        f.write("// of Y, share of the CUs with work).  Regret of the choice against the best measured shape over the\n")
         f.write(f"// {len(rows)} fitted cases: {total:.2%}; with each layer set held out of the fit in turn: {held_chosen / held_best - 1:.2%}.\n")
         f.write("#pragma once\n\nnamespace tab {\n\n")
-        f.write("constexpr int kConvShapes = 7, kConvShapeFeatures = 8;\n")
+        f.write("constexpr int kConvShapes = 7, kConvShapeFeatures = 9;\n")
         f.write("// rows x filters of the workgroup tile and workgroups a CU holds, per shape\n")
         f.write("constexpr int kConvShapeTile[kConvShapes][3] = {" + ", ".join("{%d, %d, %d}" % SHAPES[s] for s in range(7)) + "};\n")
         f.write("constexpr float kConvShapeCost[4][kConvShapes][kConvShapeFeatures] = {\n")
