@@ -98,6 +98,13 @@ RESNET18_LAYERS = [
 ]
 
 
+# (N, layer): launches of a round or two of the chip (profiled with the counters of bench.py --profile)
+MID_SIZE_LAYERS = [
+    (256, (7, 7, 512, 512, 3, 3, 1, 1, 1, 1)), (256, (14, 14, 256, 256, 3, 3, 1, 1, 1, 1)),
+    (32, (14, 14, 512, 512, 3, 3, 1, 1, 1, 1)),
+]
+
+
 def out_extent(size, pad, k, stride):
     return (size + 2 * pad - k + 1) // stride
 
@@ -332,7 +339,8 @@ def profile_sequence(torch, tab):
     """Launch sequence for counter collection: a plain 256 MiB device copy (the yardstick that
     FETCH_SIZE / WRITE_SIZE are scaled with), Quantize at the roofline shape for both bit
     widths, Conv2d (quantizer launch + conv launch) on every ResNet-18 N=16 layer, the short-K layer
-    N=256 56x56x64->64 with fp32 and with packed output, and the conv kernel of the large
+    N=256 56x56x64->64 with fp32 and with packed output, the conv kernel of three mid-size layers
+    (N=256 7x7x512->512, N=256 14x14x256->256, N=32 14x14x512->512; BNN and TNN), and the conv kernel of the large
     sweep point for all four types: the default (matrix-core) kernel, then the popcount kernel on
     the same tensors.  Three repetitions each."""
     src = torch.empty(256 * 1024 * 1024 // 4, dtype=torch.float32, device="cuda").normal_()
@@ -360,6 +368,13 @@ def profile_sequence(torch, tab):
     for _ in range(3):
         L.conv_packed_out()
     del L
+    # mid-size launches: a grid of a round or two of the chip, where one tile's serial K loop sets the duration
+    for n_batch, lay in MID_SIZE_LAYERS:
+        for type in (3, 0):
+            L = Layer(tab, torch, type, n_batch, lay, seed=11, on_device=True)
+            for _ in range(3):
+                L.conv_kernel_only()
+            del L
     for type in range(4):
         L = Layer(tab, torch, type, 256, (28, 28, 512, 512, 3, 3, 1, 1, 1, 1), seed=7, on_device=True)
         for kernel in (tab.CONV_AUTO, tab.CONV_POPCOUNT):

@@ -7,7 +7,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libtab_amd.so")
 SOURCES = ["tab_capi.hip", "tab_conv.hip", "tab_conv_mfma_tnn.hip", "tab_conv_mfma_tbn.hip", "tab_conv_mfma_btn.hip",
-           "tab_conv_mfma_bnn.hip", "tab_conv_mfma_drf.hip", "tab_conv_mfma_rtn.hip", "tab_quantize.hip"]
+           "tab_conv_mfma_bnn.hip", "tab_conv_mfma_drf.hip", "tab_conv_mfma_rtn.hip", "tab_conv_fused1x1.hip", "tab_quantize.hip"]
 OBJ_DIR = os.path.join(LIB_DIR, "obj")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -packed-fp32-ops: keep the compiler from forming packed-FP32 VALU ops from float code.

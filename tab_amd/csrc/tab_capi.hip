@@ -99,7 +99,7 @@ int tab_set_conv_kernel(int kernel, int tile)
 {
     static const int popcount_tm[4] = {7, 8, 4, 2};  // 7: the popcount kernel's own choice
     if (kernel == TAB_CONV_AUTO && tile == -1) tab::force_conv_tile(0, 0);
-    else if (kernel == TAB_CONV_MATRIX && tile >= -1 && tile <= 7) tab::force_conv_tile(9, tile);
+    else if (kernel == TAB_CONV_MATRIX && tile >= -1 && tile <= 9) tab::force_conv_tile(9, tile);
     else if (kernel == TAB_CONV_POPCOUNT && tile >= -1 && tile <= 2) tab::force_conv_tile(popcount_tm[tile + 1], 0);
     else return fail(TAB_ERR_BAD_ARGUMENT, "no conv kernel %d with tile %d", kernel, tile);
     return TAB_OK;
@@ -327,6 +327,14 @@ static int conv_from_floats(const float *dev_X, const int64_t *dev_QW, const flo
         if (e != hipSuccess) return device_fail(e, "quantize launch");
         return tab_conv2d_packed(reinterpret_cast<const int64_t *>(workspace), dev_QW, dev_btn, type, padding1, padding2, stride1,
                                  stride2, N, H, W, C, KN, KH, KW, dev_Y, stream);
+    }
+    // A small 1x1 convolution without padding: quantize and multiply in one launch, the packed activation stays in LDS
+    // (only under the automatic kernel choice: a forced kernel is what the caller wants to see run)
+    if (!tab::conv_kernel_forced() && tab::conv1x1_fused_supported(type, dev_X, C, KH, KW, padding1, padding2, s.M, KN)) {
+        hipError_t e = tab::launch_conv1x1_fused(type, dev_X, dev_ths, reinterpret_cast<const uint64_t *>(dev_QW), dev_btn, dev_Y, N, H,
+                                                 W, C, KN, stride1, stride2, s.OH, s.OW, static_cast<hipStream_t>(stream));
+        if (e != hipSuccess) return device_fail(e, "conv launch");
+        return TAB_OK;
     }
     // A 1x1 convolution with stride and no padding reads one pixel in stride1*stride2: quantize only
     // those, into a compact activation, and convolve it with stride 1 (same outputs, a fraction of

@@ -116,6 +116,12 @@ int threshold_splits(long items, long per_item);
 hipError_t launch_threshold(const float *x, long items, long per_item, float scale, float *ths, float *partial,
                             hipStream_t stream);
 
+// Quantize + 1x1 conv in one launch (tab_conv_fused1x1.hip), for calls that are bound by their launches.
+bool conv1x1_fused_supported(int type, const float *x, int C, int KH, int KW, int p1, int p2, long M, int KN);
+hipError_t launch_conv1x1_fused(int type, const float *x, const float *ths, const uint64_t *qw, const int32_t *btn, float *y, int N,
+                                int H, int W, int C, int KN, int s1, int s2, int OH, int OW, hipStream_t stream);
+
 void force_conv_tile(int tm, int ng);  // tuning hook: 0,0 restores the automatic choice
+bool conv_kernel_forced();             // true while tab_set_conv_kernel holds a choice other than the automatic one
 
 }  // namespace tab

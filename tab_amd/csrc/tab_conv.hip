@@ -342,6 +342,8 @@ void force_conv_tile(int tm, int ng)
     g_forced_kernel.store(tm == 0 ? 0 : ((tm << 8) | ((ng + 1) & 0xff)), std::memory_order_relaxed);
 }
 
+bool conv_kernel_forced() { return g_forced_kernel.load(std::memory_order_relaxed) != 0; }
+
 // fp32 accumulators hold integers up to 2^24 exactly; a product is at most 1 (9 for the 2-bit levels of
 // type 4, see conv_mfma_exact_levels) and there are 64 per word
 bool conv_mfma_exact(const ConvArgs &a) { return (long)a.G * 64 <= (1L << 22); }
@@ -411,7 +413,7 @@ hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream)
     const int force_tm = forced.tm, force_ng = forced.ng;
     if (args.qy != nullptr) {  // packed output exists in the matrix-core kernel's 64-wide shapes only
         if (!conv_mfma_exact(args)) return hipErrorInvalidValue;
-        const int shape = (force_tm == 9 && force_ng >= 0 && force_ng != 3 && force_ng <= 7) ? force_ng : conv_mfma_shape(type, args);
+        const int shape = (force_tm == 9 && force_ng >= 0 && force_ng != 3 && force_ng <= 9) ? force_ng : conv_mfma_shape(type, args);
         return launch_conv_mfma(type, args, shape, stream);
     }
     if (force_tm == 9) return launch_conv_mfma(type, args, force_ng < 0 ? conv_mfma_shape(type, args) : force_ng, stream);

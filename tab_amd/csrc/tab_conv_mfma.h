@@ -624,8 +624,10 @@ hipError_t launch_mfma_tile(ConvArgs a, hipStream_t stream)
 // Chunks of whole word pairs that stay inside a filter tap (PC even) go from global memory straight into LDS
 // (tab_conv_mfma_direct.h), measured 2-14 % faster than staging them through registers; the k-split shape keeps the piece stager of the kernel
 // above (its chunks are too short to split into pairs of words per wave, and it measured no better).
-template <int TYPE, int WM, int WN, int TM, int TN, int KCH>
+template <int TYPE, int WM, int WN, int TM, int TN, int KCH, int KS = 1, int ARUN = 0>
 hipError_t launch_mfma_direct(ConvArgs a, hipStream_t stream);
+template <int TYPE, int WM, int WN, int TM, int TN, int KS, int WORDS>
+hipError_t launch_mfma_split(const ConvArgs &a, hipStream_t stream);
 
 template <int TYPE, int WM, int WN, int TM, int TN, int KCH, int KS = 1>
 hipError_t launch_mfma_intap(const ConvArgs &a, hipStream_t stream)
@@ -674,18 +676,24 @@ hipError_t launch_mfma_regs(const ConvArgs &a, hipStream_t stream);
 // shape: 0 = 128x128, 1 = 128x64, 2 = 64x64 (rows x filters per workgroup), 3 = 32x32 with the four
 // waves splitting every chunk of four words between them, 4 = 256x64, 5 = 256x128 and 6 = 128x256
 // (eight MFMA tiles per wave: fewer operand expansions per MFMA, half the occupancy), 7 = the register-resident
-// short-K kernel (K of at most nine words; longer K falls back to the shape picked from the launch)
+// short-K kernel (K of at most nine words; longer K falls back to the shape picked from the launch),
+// 8 = 64x64 with K split over the four waves (each wave 2x2 MFMA tiles over a quarter of every chunk), 9 = 128x128 with K
+// split over two pairs of waves (each wave 2x4 MFMA tiles over half of every chunk); both need an even number of words per
+// pixel and otherwise run as shapes 2 and 0
 template <int TYPE>
 hipError_t launch_mfma_type(const ConvArgs &a, int shape, hipStream_t stream)
 {
-    if constexpr (TYPE <= 3) {
-        if (shape == 7) {
+    if (shape == 7) {
+        if constexpr (TYPE <= 3)
             if (a.G <= 9) return launch_mfma_regs<TYPE>(a, stream);
-            shape = conv_mfma_shape(TYPE, a);
-            if (shape == 7) return hipErrorInvalidValue;
-        }
+        shape = conv_mfma_shape(TYPE, a);
+        if (shape == 7) return hipErrorInvalidValue;
     }
+    if (shape == 8 && a.PC % 2 != 0) shape = 2;
+    if (shape == 9 && a.PC % 2 != 0) shape = 0;
     switch (shape) {
+    case 8: return launch_mfma_split<TYPE, 1, 1, 2, 2, 4, 2>(a, stream);
+    case 9: return launch_mfma_split<TYPE, 2, 1, 2, 4, 2, 2>(a, stream);
     case 0: return launch_mfma_shape<TYPE, 2, 2, 2, 2>(a, stream);
     case 1: return launch_mfma_shape<TYPE, 4, 1, 1, 2>(a, stream);
     case 2: return launch_mfma_shape<TYPE, 2, 2, 1, 1, true>(a, stream);

@@ -46,27 +46,54 @@ __device__ __forceinline__ int run_swizzle(int row)
     return RUN == 4 ? ((row >> 1) + (row >> 3)) & 3 : (RUN == 2 ? ((row >> 2) + (row >> 3)) & 1 : 0);
 }
 
-// PACKED: packed output (p.qy): the weights are the first MFMA operand and the epilogue packs inside a lane.
-template <int TYPE, int WM, int WN, int TM, int TN, int KCH, bool PACKED>
-__global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM * TN > 4 ? 2 : (WM * TM > 4 ? 3 : 4)))) void conv_mfma_direct(const ConvArgs p)
+// Waves per SIMD the register allocation is asked for: four with up to four MFMA tiles a wave (128 registers), three
+// with 256-row tiles (the state of more staged rows), two with eight tiles a wave.
+constexpr int direct_waves_per_eu(int type, int wm, int tm, int tn, int ks)
 {
-    static_assert(WM * WN * 64 == kConvThreads && KCH % 2 == 0, "four waves, whole pairs of words");
+    return tm * tn > 4 ? 2 : (wm * tm > 4 && ks == 1 ? 3 : 4);
+}
+
+// LDS dwords one wave deposits per 32x32 tile when KS waves exchange partial sums: 16 accumulator elements a lane as four
+// 16-byte quads, quad q of lane l at dword q * 256 + 4 * l (consecutive lanes 16 bytes apart: conflict-free 16-byte
+// accesses), then one dword a lane for BTN's count of nonzero weight bits.
+constexpr int kSplitTileDwords = 16 * 64 + 64;
+constexpr int kSplitRoundTiles = 2;  // tiles a wave deposits per exchange round (34 KB of LDS for the four waves)
+
+// PACKED: packed output (p.qy): the weights are the first MFMA operand and the epilogue packs inside a lane.
+// KS > 1: K split inside the workgroup.  The workgroup's WM x WN x KS waves form KS groups that share one
+// 32*WM*TM x 32*WN*TN tile of Y; all of them fetch every chunk together, wave group ks multiplies the pairs of words
+// ks, ks + KS, ... of each chunk, and the partial sums meet in LDS after the loop (exact in any order: they are
+// integers below 2^24).  A launch whose grid is a round or two of the chip lasts as long as one tile's serial K loop;
+// this quarters (halves) that loop for the same tile, or lets a tile of a quarter (half) the size - four (two) times
+// the workgroups to spread over the CUs - keep the large tile's ratio of operand expansions to MFMAs.  K need not be a
+// multiple of the chunk: words past it are fetched as zeros (the BNN bias counts them).
+// ARUN: granules of an activation row that neighbouring lanes fetch (0: the widest the chunk allows); a run must not
+// straddle filter taps, so layers with few words per pixel take a shorter one.
+template <int TYPE, int WM, int WN, int TM, int TN, int KCH, bool PACKED, int KS = 1, int ARUN = 0>
+__global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(direct_waves_per_eu(TYPE, WM, TM, TN, KS)))) void conv_mfma_direct(const ConvArgs p)
+{
+    static_assert(WM * WN * KS * 64 == kConvThreads && KCH % (2 * KS) == 0, "four waves, whole pairs of words per wave group");
     constexpr int PAIRS = KCH / 2;
+    constexpr int PPW = PAIRS / KS;  // pairs of words a wave multiplies per chunk
     constexpr int APL = Planes<TYPE>::A, BPL = Planes<TYPE>::B;
     constexpr int BM = 32 * WM * TM, BN = 32 * WN * TN;
     constexpr int PA = KCH * APL / 2, PB = KCH * BPL / 2;  // granules per row and chunk
     constexpr int A_GRANULES = PA * BM, B_GRANULES = PB * BN;
     constexpr int A_ITEMS = (A_GRANULES + kConvThreads - 1) / kConvThreads, B_ITEMS = (B_GRANULES + kConvThreads - 1) / kConvThreads;
     constexpr int BUF_DWORDS = 4 * (A_ITEMS + B_ITEMS) * kConvThreads;  // whole wave instructions
-    constexpr int A_RUN = granule_run(PA, APL), B_RUN = granule_run(PB, BPL);
+    constexpr int A_RUN = ARUN ? ARUN : granule_run(PA, APL), B_RUN = granule_run(PB, BPL);
     static_assert(BM % 64 == 0 && BN % 64 == 0, "one wave instruction moves 64 / RUN rows of one run");
+    static_assert(PA % A_RUN == 0, "whole runs");
+    // partial sums of the KS wave groups: kSplitRoundTiles tiles per wave and round, then the packed epilogue's 32 dwords a wave
+    constexpr int SPLIT_DWORDS = KS > 1 ? (kConvThreads / 64) * (kSplitRoundTiles * kSplitTileDwords + 32) : 0;
 
-    __shared__ __attribute__((aligned(16))) uint32_t lds[2 * BUF_DWORDS];
+    __shared__ __attribute__((aligned(16))) uint32_t lds[2 * BUF_DWORDS > SPLIT_DWORDS ? 2 * BUF_DWORDS : SPLIT_DWORDS];
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int r = lane & 31, kb = lane >> 5;
-    const int wm = wave % WM, wn = wave / WM;
+    const int ks = wave / (WM * WN), wsub = wave % (WM * WN);  // wave group along K, wave inside the group
+    const int wm = wsub % WM, wn = wsub / WM;
     const int pixels = p.OH * p.OW;
     const size_t image_words = (size_t)p.H * p.W * p.PC * APL;
     const size_t filter_bytes = (size_t)p.G * BPL * 8;
@@ -78,6 +105,7 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
     // ---- what this lane fetches: granule idx = tid + i * 256 = (run * ROWS + row) * RUN + column ------
     int ih0[A_ITEMS], iw0[A_ITEMS];
     uint32_t a_base[A_ITEMS], b_base[B_ITEMS];
+    int b_word[KS > 1 ? B_ITEMS : 1];  // KS > 1: first word of the lane's granule inside a chunk (words past K are zeros)
     const int n_first = (int)div32((uint32_t)m0, p.div_pixels);  // uniform
     const size_t a_bytes = (size_t)(p.N - n_first) * image_words * 8;
     const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(p.qx + (size_t)n_first * image_words), 0,
@@ -109,6 +137,7 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
         const int granule = idx / B_RUN / BN * B_RUN + ((idx % B_RUN - run_swizzle<B_RUN>(row & 15)) & (B_RUN - 1));
         const bool live = granule < PB && (n0 + row) < p.KN;
         b_base[i] = live ? (uint32_t)row * (uint32_t)filter_bytes + (uint32_t)granule * 16u : kNoFilter;
+        if (KS > 1) b_word[i] = granule * (BPL == 1 ? 2 : 1);
     }
     // chunk `chunk` into buf; !live_chunk: zeros (every offset out of range)
     auto fetch = [&](int chunk, uint32_t *buf, bool live_chunk) {
@@ -122,14 +151,16 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
             const int kh = (int)fastdiv(tap, p.div_kw);
             const int kw = (int)tap - kh * p.KW;
             const uint32_t tap_off = (uint32_t)((kh * p.W + kw) * p.PC + pc) * (uint32_t)(APL * 8);
-            const bool ok = live_chunk && (unsigned)(ih0[i] + kh) < (unsigned)p.H && (unsigned)(iw0[i] + kw) < (unsigned)p.W;
+            // (KS > 1: the last chunk may reach past K; a run lies inside a tap, hence on one side of the end of K)
+            const bool ok = live_chunk && (KS == 1 || g < p.G) && (unsigned)(ih0[i] + kh) < (unsigned)p.H && (unsigned)(iw0[i] + kw) < (unsigned)p.W;
             load16_to_lds(a_rsrc, buf + 4 * (i * kConvThreads + wave * 64), ok ? a_base[i] + tap_off : kNoData);
         }
         const uint32_t word_off = (uint32_t)g0 * (uint32_t)(BPL * 8);
 #pragma unroll
         for (int i = 0; i < B_ITEMS; i++)
             load16_to_lds(b_rsrc, buf + 4 * ((A_ITEMS + i) * kConvThreads + wave * 64),
-                          b_base[i] == kNoFilter || !live_chunk ? kNoFilter : b_base[i] + word_off);
+                          b_base[i] == kNoFilter || !live_chunk || (KS > 1 && g0 + b_word[i % (KS > 1 ? B_ITEMS : 1)] >= p.G)
+                              ? kNoFilter : b_base[i] + word_off);
     };
 
     const ExpandConsts consts;
@@ -151,22 +182,24 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
     constexpr int B_REGION = 4 * A_ITEMS * kConvThreads;
 
     constexpr int HS = TYPE == 5 ? 1 : 2;  // MFMA steps per pair of words: one per half, type 5 both halves at once
-    constexpr int STEPS = PAIRS * HS;
+    constexpr int STEPS = PPW * HS;
     // (with one expansion or more per MFMA the vector unit is the limit either way and the pinned order only costs)
     constexpr bool PIPELINED = TYPE != 5 && TM * TN >= 8;
     constexpr int NM = TM * TN, NE = TM + TN;
     uint32_t a_w[2][TM][2 * APL], b_w[2][TN][2 * BPL];  // [low half, high half] of every plane of the lane's word
-    auto read_pair = [&](const uint32_t *buf, int pair) {
+    // the wave's pair j of a chunk (pair ks + KS * j of the chunk) into register set j & 1
+    auto read_pair = [&](const uint32_t *buf, int j) {
+        const int pair = KS == 1 ? j : ks + KS * j;
 #pragma unroll
         for (int mt = 0; mt < TM; mt++) {
             const uint32_t *src = buf + lane_part(APL, A_RUN, BM, a_row, a_sw, pair) + mt * 32 * A_RUN * 4;
             if (APL == 1) {
                 const u32x2 v = *reinterpret_cast<const u32x2 *>(src);
-                a_w[pair & 1][mt][0] = v[0]; a_w[pair & 1][mt][1] = v[1];
+                a_w[j & 1][mt][0] = v[0]; a_w[j & 1][mt][1] = v[1];
             } else {
                 const u32x4 v = *reinterpret_cast<const u32x4 *>(src);
 #pragma unroll
-                for (int e = 0; e < 4; e++) a_w[pair & 1][mt][e] = v[e];
+                for (int e = 0; e < 4; e++) a_w[j & 1][mt][e] = v[e];
             }
         }
 #pragma unroll
@@ -174,11 +207,11 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
             const uint32_t *src = buf + B_REGION + lane_part(BPL, B_RUN, BN, b_row, b_sw, pair) + nt * 32 * B_RUN * 4;
             if (BPL == 1) {
                 const u32x2 v = *reinterpret_cast<const u32x2 *>(src);
-                b_w[pair & 1][nt][0] = v[0]; b_w[pair & 1][nt][1] = v[1];
+                b_w[j & 1][nt][0] = v[0]; b_w[j & 1][nt][1] = v[1];
             } else {
                 const u32x4 v = *reinterpret_cast<const u32x4 *>(src);
 #pragma unroll
-                for (int e = 0; e < 4; e++) b_w[pair & 1][nt][e] = v[e];
+                for (int e = 0; e < 4; e++) b_w[j & 1][nt][e] = v[e];
             }
         }
     };
@@ -234,7 +267,6 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
             for (int e = 0; e < 16; e++) acc[mt][nt][e] = 0.f;
 #pragma unroll
     for (int nt = 0; nt < TN; nt++) b_nonzero[nt] = 0;
-
     fetch(0, lds, true);
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
@@ -261,7 +293,7 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
                     __builtin_amdgcn_s_waitcnt(0);  // this wave's part of the next chunk has landed
                     __syncthreads();
                     read_pair(next, 0);
-                } else if (h == 0 && pair + 1 < PAIRS) {
+                } else if (h == 0 && pair + 1 < PPW) {
                     read_pair(buf, pair + 1);
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -288,8 +320,8 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
             if (more) fetch(chunk + 1, next, true);
             read_pair(buf, 0);
 #pragma unroll
-            for (int pair = 0; pair < PAIRS; pair++) {
-                if (pair + 1 < PAIRS) read_pair(buf, pair + 1);
+            for (int pair = 0; pair < PPW; pair++) {
+                if (pair + 1 < PPW) read_pair(buf, pair + 1);
 #pragma unroll
                 for (int h = 0; h < HS; h++) {
                     i32x8 a_op[TM], b_op[TN];
@@ -321,9 +353,56 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
             __syncthreads();
         }
     }
-
     scale_ternary_sums<TYPE>(acc);
-    if constexpr (PACKED) {
+    if constexpr (KS > 1) {
+        // The KS groups hold partial sums of the same tiles.  Rounds of kSplitRoundTiles tiles: every wave deposits its
+        // part of the round's tiles (and BTN's partial count of nonzero weight bits), the wave group (round's tile) % KS
+        // of each wave position adds the KS parts of one tile and finishes it like a wave that owned it alone.
+        constexpr int NT = TM * TN, RT = kSplitRoundTiles;
+        static_assert(NT % RT == 0, "whole rounds");
+        float *parts = reinterpret_cast<float *>(lds);
+        uint32_t *exchange = lds + (kConvThreads / 64) * RT * kSplitTileDwords + wave * 32;
+        __syncthreads();  // the operand buffers are free: every wave has read its last pair
+#pragma unroll
+        for (int round = 0; round < NT / RT; round++) {
+#pragma unroll
+            for (int i = 0; i < RT; i++) {
+                const int t = round * RT + i, mt = t / TN, nt = t % TN;
+                float *dst = parts + (wave * RT + i) * kSplitTileDwords;
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+                    *reinterpret_cast<f32x4 *>(dst + q * 256 + lane * 4) =
+                        f32x4{acc[mt][nt][4 * q], acc[mt][nt][4 * q + 1], acc[mt][nt][4 * q + 2], acc[mt][nt][4 * q + 3]};
+                if (TYPE == 2) dst[16 * 64 + lane] = __int_as_float(b_nonzero[nt]);
+            }
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < RT; i++) {
+                const int t = round * RT + i, mt = t / TN, nt = t % TN;
+                if (ks != t % KS) continue;  // wave-uniform
+                f32x16 sum[1][1];
+                int nonzero[1] = {0};
+#pragma unroll
+                for (int e = 0; e < 16; e++) sum[0][0][e] = 0.f;
+#pragma unroll
+                for (int k = 0; k < KS; k++) {
+                    const float *src = parts + ((k * (WM * WN) + wsub) * RT + i) * kSplitTileDwords;
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        const f32x4 v = *reinterpret_cast<const f32x4 *>(src + q * 256 + lane * 4);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) sum[0][0][4 * q + e] += v[e];
+                    }
+                    if (TYPE == 2) nonzero[0] += __float_as_int(src[16 * 64 + lane]);
+                }
+                if constexpr (PACKED)
+                    conv_mfma_epilogue_packed<TYPE, 1, 1, KCH>(p, sum, nonzero, wave_m0 + mt * 32, wave_n0 + nt * 32, lane, exchange);
+                else
+                    conv_mfma_epilogue<TYPE, 1, 1, KCH, 1, false>(p, sum, nonzero, wave_m0 + mt * 32, wave_n0 + nt * 32, lane, 0, nullptr);
+            }
+            if (round + 1 < NT / RT) __syncthreads();  // the parts are read before the next round overwrites them
+        }
+    } else if constexpr (PACKED) {
         // BTN hands its biases round through LDS: not before every wave has read its last operands (the pipelined
         // loop reads the zeros past the last chunk after the chunk's barrier and counts their nonzero weights)
         if (TYPE == 2) __syncthreads();
@@ -333,27 +412,45 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM
     }
 }
 
-template <int TYPE, int WM, int WN, int TM, int TN, int KCH>
+template <int TYPE, int WM, int WN, int TM, int TN, int KCH, int KS, int ARUN>
 hipError_t launch_mfma_direct(ConvArgs a, hipStream_t stream)
 {
     constexpr int BM = 32 * WM * TM, BN = 32 * WN * TN;
     // words of a run of activation granules, which must not straddle filter taps
-    constexpr int A_RUN_WORDS = granule_run(KCH * Planes<TYPE>::A / 2, Planes<TYPE>::A) * (Planes<TYPE>::A == 1 ? 2 : 1);
-    if (a.G % KCH != 0 || a.PC % A_RUN_WORDS != 0) return hipErrorInvalidValue;
+    constexpr int A_RUN_WORDS = (ARUN ? ARUN : granule_run(KCH * Planes<TYPE>::A / 2, Planes<TYPE>::A)) * (Planes<TYPE>::A == 1 ? 2 : 1);
+    if ((KS == 1 && a.G % KCH != 0) || a.PC % A_RUN_WORDS != 0) return hipErrorInvalidValue;
     a.kcw = KCH;
-    a.nchunks = a.G / KCH;
+    a.nchunks = (a.G + KCH - 1) / KCH;  // the split-K kernels fetch the words past K as zeros
     a.tiles_m = (a.M + BM - 1) / BM;
     const long blocks = order_workgroups<Planes<TYPE>::A>(a, (a.KN + BN - 1) / BN);
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
     if (a.qy != nullptr) {
         if constexpr (TYPE <= 3)
-            conv_mfma_direct<TYPE, WM, WN, TM, TN, KCH, true><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
+            conv_mfma_direct<TYPE, WM, WN, TM, TN, KCH, true, KS, ARUN><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
         else
             return hipErrorInvalidValue;  // no packed output for types 4 and 5
     } else {
-        conv_mfma_direct<TYPE, WM, WN, TM, TN, KCH, false><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
+        conv_mfma_direct<TYPE, WM, WN, TM, TN, KCH, false, KS, ARUN><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
     }
     return hipGetLastError();
+}
+
+// Split-K launch: chunk length and run of activation granules from the layer's words per pixel.  WORDS = words every
+// wave group multiplies per chunk.  False (nothing launched) when the layer's words per pixel fit no run.
+template <int TYPE, int WM, int WN, int TM, int TN, int KS, int WORDS>
+hipError_t launch_mfma_split(const ConvArgs &a, hipStream_t stream)
+{
+    constexpr int APL = Planes<TYPE>::A;
+    constexpr int KCH = KS * WORDS;
+    constexpr int PA = KCH * APL / 2;
+    // granules of 16 bytes: two words of a one-plane activation, one word of a two-plane one
+    const int granules_per_pixel = a.PC * APL / 2;  // PC is even here
+    if (a.PC % 2 != 0) return hipErrorInvalidValue;
+    if constexpr (PA % 4 == 0)
+        if (granules_per_pixel % 4 == 0) return launch_mfma_direct<TYPE, WM, WN, TM, TN, KCH, KS, 4>(a, stream);
+    if constexpr (PA % 2 == 0)
+        if (granules_per_pixel % 2 == 0) return launch_mfma_direct<TYPE, WM, WN, TM, TN, KCH, KS, 2>(a, stream);
+    return launch_mfma_direct<TYPE, WM, WN, TM, TN, KCH, KS, 1>(a, stream);
 }
 
 }  // namespace
