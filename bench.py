@@ -45,20 +45,22 @@ HEADLINE_REPS = 7      # repetitions of the timed `steps` loop; the median is re
 TRAFFIC_PROFILE = os.path.join("profiles", "quantize_conv_profile_sequence_traffic.txt")
 
 
-def profiled_step_traffic():
-    """(bytes, source) of the measured HBM traffic of one step's conv launches, read from the tracked profile summary;
-    (None, reason) when the file or the line is missing."""
+def profiled_figure(name):
+    """(value, source) of a figure the tracked profile summary states on a line "<name> = <integer>"; (None, reason) when
+    the file or the line is missing.  conv_step_traffic_bytes: measured HBM traffic of one step's conv-side launches;
+    conv_step_trace_ns / step_trace_ns: sum over one step's conv-side / all launches of the average duration in the
+    rocprofv3 kernel trace."""
     import re
 
     path = os.path.join(ROOT, TRAFFIC_PROFILE)
     try:
         for number, line in enumerate(open(path), 1):
-            m = re.match(r"\s*conv_step_traffic_bytes\s*=\s*(\d+)", line)
+            m = re.match(r"\s*" + name + r"\s*=\s*(\d+)", line)
             if m:
                 return int(m.group(1)), f"{TRAFFIC_PROFILE}:{number}"
     except OSError:
         return None, f"{TRAFFIC_PROFILE} not found"
-    return None, f"{TRAFFIC_PROFILE} has no conv_step_traffic_bytes line"
+    return None, f"{TRAFFIC_PROFILE} has no {name} line"
 
 
 def valu_peak_tops(type):
@@ -151,6 +153,22 @@ class Layer:
 
     def conv2d(self):
         return self.tab.Conv2d(self.x, self.QW, self.x_ths, self.BTN, *self.args)
+
+    def launches(self):
+        """Kernels one conv2d() enqueues: 2 (quantizer, conv) or 1 (small 1x1 layers: quantize + conv in one kernel)."""
+        return self.tab.conv2d_launches(self.x, *self.args)
+
+    def conv_side_launch(self):
+        """The launch of conv2d() that multiplies: the conv kernel on the packed activation, or the whole call where
+        quantizer and conv are one kernel."""
+        return self.conv2d() if self.launches() == 1 else self.conv_kernel_only()
+
+    def conv_side_bytes(self):
+        """Algorithmic HBM bytes of that launch: packed activation (or, in one launch with the quantizer, the fp32 pixels
+        it reads) + weights + fp32 Y."""
+        if self.launches() == 1:
+            return layer_bytes(self.N, self.layer, self.wbits)
+        return conv_kernel_bytes(self.N, self.layer, self.abits, self.wbits)
 
     def conv_kernel_only(self):
         return self.tab.Conv2dPacked(self.QX, self.QW, self.BTN, *self.args)
@@ -338,7 +356,8 @@ def reference_gemm_baseline(oracle, L, budget_s=3.0):
 def profile_sequence(torch, tab):
     """Launch sequence for counter collection: a plain 256 MiB device copy (the yardstick that
     FETCH_SIZE / WRITE_SIZE are scaled with), Quantize at the roofline shape for both bit
-    widths, Conv2d (quantizer launch + conv launch) on every ResNet-18 N=16 layer, the short-K layer
+    widths, Conv2d on every ResNet-18 N=16 layer (quantizer launch + conv launch, or the one launch that does both on
+    the 1x1 layers; bracketed by two threshold launches as markers), the short-K layer
     N=256 56x56x64->64 with fp32 and with packed output, the conv kernel of three mid-size layers
     (N=256 7x7x512->512, N=256 14x14x256->256, N=32 14x14x512->512; BNN and TNN), and the conv kernel of the large
     sweep point for all four types: the default (matrix-core) kernel, then the popcount kernel on
@@ -357,10 +376,15 @@ def profile_sequence(torch, tab):
         tab.Quantize(xq, ths, 2, qN, qH, qW, qC)
     del xq
     layers = [Layer(tab, torch, 3, 16, l, seed=i) for i, l in enumerate(RESNET18_LAYERS)]
+    marker = torch.ones(64, device="cuda")
     torch.cuda.synchronize()
+    # the launches of the headline step, three times over, between two marker launches (the threshold kernels, which
+    # nothing else in this sequence runs) that tell a reader of the trace where they start and end
+    tab.Threshold(marker, 1, 1.0)
     for L in layers:
         for _ in range(3):
             L.conv2d()
+    tab.Threshold(marker, 1, 1.0)
     del layers
     L = Layer(tab, torch, 3, 256, RESNET18_LAYERS[0], seed=0, on_device=True)
     for _ in range(3):
@@ -492,21 +516,26 @@ def main():
     packed_steps = max(1, args.steps // per_graph) * per_graph
 
     # ---- per layer: latency of the whole call, kernel-only rates -------------------------
-    per_layer, conv_ops, conv_ms = [], 0, 0.0
+    per_layer, conv_ops, conv_ms, step_launches = [], 0, 0.0, 0
     for l in layers:
         call_ms = graph_time_ms(torch, l.conv2d, 20)
-        k_ms = graph_time_ms(torch, l.conv_kernel_only, 20)
-        q_ms = graph_time_ms(torch, l.quantize_only, 20)
+        fused = l.launches() == 1
+        k_ms = call_ms if fused else graph_time_ms(torch, l.conv_kernel_only, 20)
+        q_ms = None if fused else graph_time_ms(torch, l.quantize_only, 20)
         conv_ops += l.ops
         conv_ms += k_ms
-        kb = conv_kernel_bytes(N, l.layer)
-        per_layer.append({"layer": layer_name(N, l.layer), "latency_us": round(call_ms * 1e3, 2),
-                          "conv_kernel_us": round(k_ms * 1e3, 2), "quantize_kernel_us": round(q_ms * 1e3, 2),
+        step_launches += l.launches()
+        kb = l.conv_side_bytes()
+        per_layer.append({"layer": layer_name(N, l.layer), "launches": l.launches(), "latency_us": round(call_ms * 1e3, 2),
+                          "conv_kernel_us": round(k_ms * 1e3, 2),
+                          "quantize_kernel_us": None if fused else round(q_ms * 1e3, 2),
                           "conv_kernel_tops": round(l.ops / k_ms / 1e9, 2),
                           "frac_mfma_peak": round(l.ops / k_ms / 1e9 / MFMA_FP4_PEAK_TOPS, 4),
+                          "over_valu_planning_peak": round(l.ops / k_ms / 1e9 / planning_peak_tops(3), 4),
                           "conv_kernel_hbm_floor_us": round(kb / HBM_PEAK_GBS / 1e3, 2),
+                          "conv_kernel_frac_of_hbm_peak": round(kb / HBM_PEAK_GBS / 1e3 / (k_ms * 1e3), 4),
                           "hbm_floor_us": round(layer_bytes(N, l.layer) / HBM_PEAK_GBS / 1e3, 2)})
-    achieved = conv_ops / conv_ms / 1e9  # TOP/s over the conv launches of one step
+    achieved = conv_ops / conv_ms / 1e9  # TOP/s over the conv-side launches of one step, HIP events
     # the same launches with the popcount kernel, for the comparison the matrix-core kernel has to win
     tab.set_conv_kernel(tab.CONV_POPCOUNT, -1)
     popcount_ms = sum(graph_time_ms(torch, l.conv_kernel_only, 20) for l in layers)
@@ -514,38 +543,65 @@ def main():
     # Which roof bounds these launches: arithmetic intensity (binary ops per algorithmic HBM byte) against
     # the ridge of the two published peaks.  At N=16 every layer lies below it (the fp32 Y dominates the
     # bytes), so the bound of record is HBM; the matrix-core fraction is kept beside it.
-    conv_bytes = sum(conv_kernel_bytes(N, l.layer) for l in layers)
+    conv_bytes = sum(l.conv_side_bytes() for l in layers)
     intensity = conv_ops / conv_bytes
     ridge = MFMA_FP4_PEAK_TOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
-    achieved_gbs = conv_bytes / conv_ms / 1e6
     hbm_bound = intensity < ridge
-    traffic, traffic_source = profiled_step_traffic()
-    roofline = {"kernel": "conv_mfma_direct<BNN> / conv_mfma<BNN> (v_mfma_f32_32x32x64_f8f6f4, FP4 operands)",
+    traffic, traffic_source = profiled_figure("conv_step_traffic_bytes")
+    # Durations: the sum over the ten launches of their average duration in the rocprofv3 kernel trace of
+    # `bench.py --profile` (a tracked summary, like `traffic`): launches timed back to back with HIP events overlap the
+    # tail of one with the head of the next and read some 10 % shorter, so the trace is the figure of record and the live
+    # HIP-event figure stands beside it.  Without the summary the live figure is all there is.
+    trace_ns, trace_source = profiled_figure("conv_step_trace_ns")
+    step_trace_ns, step_trace_source = profiled_figure("step_trace_ns")
+    record_ms = trace_ns / 1e6 if trace_ns else conv_ms
+    record_tops = conv_ops / record_ms / 1e9
+    record_gbs = conv_bytes / record_ms / 1e6
+    step_bytes = sum(layer_bytes(N, l.layer) for l in layers)
+    fused_layers = sum(1 for l in layers if l.launches() == 1)
+    roofline = {"kernel": f"the {len(layers)} conv-side launches of one step: {len(layers) - fused_layers}x conv_mfma_direct<BNN> / conv_mfma<BNN> "
+                          f"and {fused_layers}x conv1x1_fused<BNN> (v_mfma_f32_32x32x64_f8f6f4, FP4 operands)",
                 "bound": "hbm" if hbm_bound else "mfma",
-                "achieved": round(achieved_gbs if hbm_bound else achieved, 2),
+                "achieved": round(record_gbs if hbm_bound else record_tops, 2),
                 "peak": HBM_PEAK_GBS if hbm_bound else MFMA_FP4_PEAK_TOPS,
                 "unit": "GB/s" if hbm_bound else "TFLOP/s",
-                "frac": round(achieved_gbs / HBM_PEAK_GBS if hbm_bound else achieved / MFMA_FP4_PEAK_TOPS, 4),
+                "frac": round(record_gbs / HBM_PEAK_GBS if hbm_bound else record_tops / MFMA_FP4_PEAK_TOPS, 4),
+                "durations_from": trace_source if trace_ns else "HIP events of this run (no tracked kernel-trace figure found)",
+                "sum_of_launch_durations_us": round(record_ms * 1e3, 2),
+                "hip_events": {"sum_of_launch_durations_us": round(conv_ms * 1e3, 2),
+                               "achieved": round(conv_bytes / conv_ms / 1e6 if hbm_bound else achieved, 2),
+                               "frac": round(conv_bytes / conv_ms / 1e6 / HBM_PEAK_GBS if hbm_bound else achieved / MFMA_FP4_PEAK_TOPS, 4),
+                               "note": "the same launches timed in this run: HIP events around graph replays of 20 back-to-back "
+                                       "launches per layer"},
                 "traffic": traffic, "traffic_source": traffic_source,
                 "algorithmic_bytes": conv_bytes,
-                "launches": len(layers), "sum_of_launch_durations_us": round(conv_ms * 1e3, 2),
+                "launches": len(layers),
                 "ops_per_byte": round(intensity, 1), "ridge_ops_per_byte": round(ridge, 1),
-                "mfma_achieved_tops": round(achieved, 2), "mfma_peak_tops": MFMA_FP4_PEAK_TOPS,
-                "mfma_frac": round(achieved / MFMA_FP4_PEAK_TOPS, 4),
-                "popcount_kernel_achieved_tops": round(conv_ops / popcount_ms / 1e9, 2),
-                "valu_popcount_planning_peak": round(planning_peak_tops(3), 1),
-                "achieved_over_valu_planning_peak": round(achieved / planning_peak_tops(3), 4),
-                "note": "the ten conv launches of one step: achieved = their algorithmic HBM bytes (packed activation + "
-                        "weights + fp32 Y) / the sum of their average durations (HIP events around graph replays of 20 "
-                        "launches per layer); bound = hbm because their ops per byte lie below the ridge of the published "
-                        "peaks (FP4 MFMA 10.1 PFLOP/s, one effective binary op = one FP4 flop; HBM 8 TB/s); mfma_* give "
-                        "the same launches against the matrix-core peak.  At N=16 every launch is a few microseconds, "
-                        "launch- and latency-bound (see resnet18_bnn_N256 and sweep_N256_28x28x512_3x3 for kernels long "
-                        "enough to load the matrix cores, quantize for the HBM-bound kernel at its roofline shape); "
-                        "traffic = rocprofv3 FETCH_SIZE + WRITE_SIZE of the same ten launches, scaled by a copy, read from "
-                        "the tracked profile summary named in traffic_source (a separate profiler run, not this run); "
-                        "popcount_kernel_achieved_tops is the VALU popcount kernel on the same launches, "
-                        "valu_popcount_planning_peak its roofline (256 CU x 64 lanes x 2.4 GHz / 2 lane-ops per pair)"}
+                # the roofline the benchmark specification names for conv: VALU popcount, 256 CU x 64 lanes x 2.4 GHz over
+                # the reference's two lane-ops per word pair (BNN); target: at least half of it on these layers
+                "valu_popcount_roofline_of_record": {"achieved_tops": round(record_tops, 2), "peak_tops": round(planning_peak_tops(3), 1),
+                                                     "frac": round(record_tops / planning_peak_tops(3), 4), "target_frac": 0.5,
+                                                     "frac_hip_events": round(achieved / planning_peak_tops(3), 4),
+                                                     "popcount_kernel_achieved_tops": round(conv_ops / popcount_ms / 1e9, 2)},
+                "mfma": {"achieved_tops": round(record_tops, 2), "peak_tops": MFMA_FP4_PEAK_TOPS,
+                         "frac": round(record_tops / MFMA_FP4_PEAK_TOPS, 4)},
+                # the whole step against HBM: every launch of the ten calls (quantizers included), the bytes a call has to
+                # move (fp32 X, packed weights, fp32 Y)
+                "whole_step": {"launches": step_launches, "algorithmic_bytes": step_bytes,
+                               "ms_per_step": round(ms_per_step, 4),
+                               "achieved_GBps": round(step_bytes / ms_per_step / 1e6, 1),
+                               "frac_hbm_peak": round(step_bytes / ms_per_step / 1e6 / HBM_PEAK_GBS, 4),
+                               "kernel_trace_sum_us": round(step_trace_ns / 1e3, 2) if step_trace_ns else None,
+                               "kernel_trace_source": step_trace_source},
+                "note": "the ten conv-side launches of one step (for the three 1x1 layers quantizer and conv are one kernel and "
+                        "the launch reads the fp32 pixels): achieved = their algorithmic HBM bytes / the sum of their average "
+                        "durations in the rocprofv3 kernel trace named in durations_from (a separate profiler run of "
+                        "`bench.py --profile`, as for traffic); hip_events = the same launches timed in this run; bound = hbm "
+                        "because their ops per byte lie below the ridge of the published peaks (FP4 MFMA 10.1 PFLOP/s, one "
+                        "effective binary op = one FP4 flop; HBM 8 TB/s).  At N=16 every launch is a few microseconds, launch- "
+                        "and latency-bound (see resnet18_bnn_N256 and sweep_N256_28x28x512_3x3 for kernels long enough to load "
+                        "the matrix cores, quantize for the HBM-bound kernel at its roofline shape); traffic = rocprofv3 "
+                        "FETCH_SIZE + WRITE_SIZE of the same launches, scaled by a copy"}
 
     def rate(times_s, steps):
         return {"tops": round(total_ops * steps / median_of(times_s) / 1e12, 3),
@@ -558,7 +614,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": "BNN (type 3) ResNet-18 layer set, N=16: 4x 3x3 s1 + 3x 3x3 s2 + 3x 1x1 s2; "
                                "one step = Conv2d (quantize + conv) on all 10 layers; ten steps per HIP graph replay",
-                   "binary_ops_per_step": total_ops},
+                   "binary_ops_per_step": total_ops, "kernel_launches_per_step": step_launches},
         "timing": {"repetitions": len(times), "value_is": "median repetition of the timed steps loop",
                    "ms_per_step_min": round(min(times) / args.steps * 1e3, 4),
                    "ms_per_step_max": round(max(times) / args.steps * 1e3, 4),

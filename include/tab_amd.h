@@ -71,7 +71,9 @@ int tab_out_extent(int in, int pad, int k, int stride);
  *   dev_QX   int64 [N*H*W*PC*bitwidth], aligned to a whole packed element (8*bitwidth bytes; the same holds
  *            for tab_quantize_nchw, 16 bytes for tab_quantize_format); every element is written
  *   dev_BTN  int32 [N]; bitwidth 2: popcount of item n's nonzero plane (TAB_GEMM.cu:150-160,
- *            for every n); bitwidth 1: zeros (TAB_GEMM.cu:283)
+ *            for every n); bitwidth 1: zeros (TAB_GEMM.cu:283).  NULL: not wanted (an activation's
+ *            counts are read by nobody); the launches that produce them are then skipped.  The same
+ *            holds for tab_quantize_nchw.
  */
 int tab_quantize(const float *dev_X, const float *dev_ths, int bitwidth, int N, int H, int W,
                  int C, int64_t *dev_QX, int32_t *dev_BTN, void *stream);
@@ -112,6 +114,8 @@ int tab_quantize_format(const float *dev_X, const float *dev_ths, int type, int 
 size_t tab_threshold_workspace_bytes(int N, long per_item);
 int tab_threshold(const float *dev_X, int N, long per_item, float scale, float *dev_ths,
                   void *workspace, size_t workspace_bytes, void *stream);
+int tab_conv2d_launches(const float *dev_X, int type, int padding1, int padding2, int stride1, int stride2,
+                        int N, int H, int W, int C, int KN, int KH, int KW);
 
 /*
  * Bytes of device scratch tab_conv2d needs for the packed activation
@@ -138,6 +142,10 @@ size_t tab_conv2d_workspace_bytes(int type, int N, int H, int W, int C);
  * Types 4 and 5 (CPU-only in the reference, TAB_CPU.cpp:507-614) are accepted too: X goes through
  * tab_quantize_format, dev_QW holds the same format, zero words are the value 0, and Y is
  * DRFGEMM_baseline's / RTNGEMM_baseline's integer as fp32.  Type 4 needs 9 * 64 * K words < 2^24.
+ * Launches: the quantizer, then the fused pad + im2row + GEMM kernel; a small 1x1 convolution without
+ * padding (64, 128, 256 or 512 channels, types 0..3) quantizes and multiplies in ONE kernel and leaves
+ * the workspace untouched.  tab_conv2d_launches() says which (1 or 2; 0 on bad arguments), for tools that
+ * attribute time per launch; dev_X matters only through its alignment.
  */
 int tab_conv2d(const float *dev_X, const int64_t *dev_QW, const float *dev_ths,
                const int32_t *dev_btn, int type, int padding1, int padding2, int stride1,
@@ -198,12 +206,16 @@ int tab_conv2d_packed_out(const int64_t *dev_QX, const int64_t *dev_QW, const in
 /*
  * Which kernel tab_conv2d / tab_conv2d_packed launch.  Both give bit-identical Y; the switch exists
  * for verification and tuning and has no counterpart in the reference (which has one GEMM kernel
- * per type, TAB_GEMM.cu:25-147).  Process-wide, not thread-safe against concurrent conv calls.
+ * per type, TAB_GEMM.cu:25-147).  Process-wide: the choice is one atomic word, a conv call on another
+ * thread sees either the old or the new choice.  While a choice other than TAB_CONV_AUTO is held,
+ * tab_conv2d always runs the quantizer and the chosen conv kernel as two launches.
  *   TAB_CONV_AUTO      (tile -1) the library's choice: matrix cores, tile picked from the shape
  *   TAB_CONV_MATRIX    bit planes expanded to FP4 operands of v_mfma_f32_32x32x64_f8f6f4;
  *                      tile 0: 128x128, 1: 128x64, 2: 64x64, 3: 32x32 with K split over the
  *                      four waves, 4: 256x64, 5: 256x128, 6: 128x256, 7: weights resident in registers
- *                      (K of at most nine words; longer K takes the library's choice); -1: picked from the shape
+ *                      (K of at most nine words; longer K takes the library's choice), 8: 64x64 and
+ *                      9: 128x128 with K split over four / two groups of waves inside the workgroup (an
+ *                      even number of words per pixel; otherwise tiles 2 and 0); -1: picked from the shape
  *   TAB_CONV_POPCOUNT  the reference's xor/and + popcount formulation on the vector ALU;
  *                      tile 0: big, 1: medium, 2: small; -1: picked from the shape
  *                      (types 4 and 5 exist on the matrix cores only and ignore this choice)

@@ -85,6 +85,34 @@ def Quantize(X, thresholds, bitwidth, N, H, W, C):
     return [QX, BTN]
 
 
+def QuantizeActivation(X, thresholds, bitwidth, N, H, W, C, nchw=False):
+    """QX of Quantize (or, with nchw, of QuantizeNCHW with X given as N, C, H, W) without the BTN vector: an
+    activation's counts are read by nobody, and passing NULL for them to the C ABI skips the launches that
+    produce them."""
+    _check_input(X, "X")
+    _check_input(thresholds, "thresholds")
+    _check_dtype(X, torch.float32, "X")
+    _check_dtype(thresholds, torch.float32, "thresholds")
+    bitwidth, N, H, W, C = int(bitwidth), int(N), int(H), int(W), int(C)
+    if bitwidth not in (1, 2):
+        raise RuntimeError(f"bitwidth must be 1 or 2, got {bitwidth}")
+    if min(N, H, W, C) < 1:
+        raise RuntimeError("N, H, W, C must be positive")
+    if X.numel() != N * H * W * C:
+        raise RuntimeError(f"X has {X.numel()} elements, expected N*H*W*C = {N * H * W * C}")
+    if thresholds.numel() < N:
+        raise RuntimeError(f"thresholds has {thresholds.numel()} elements, expected at least N = {N}")
+    if thresholds.device != X.device:
+        raise RuntimeError("X and thresholds must be on the same device")
+    with torch.cuda.device(X.device):
+        QX = torch.empty((N, H, W, packed_channels(C), bitwidth), dtype=torch.int64, device=X.device)
+        if nchw:
+            _capi.check(_lib, _lib.tab_quantize_nchw(X.data_ptr(), thresholds.data_ptr(), bitwidth, N, C, H, W, QX.data_ptr(), None, _stream()))
+        else:
+            _capi.check(_lib, _lib.tab_quantize(X.data_ptr(), thresholds.data_ptr(), bitwidth, N, H, W, C, QX.data_ptr(), None, _stream()))
+    return QX
+
+
 def QuantizeNCHW(X, thresholds, bitwidth, N, C, H, W):
     """Quantize on an NCHW fp32 tensor (the layout the reference's CPU quantizers read, TAB_CPU.cpp:20-206, and
     the argument order of its CPU binding, TAB_CPU.cpp:621): returns [QX, BTN] exactly as
@@ -208,6 +236,11 @@ def Conv2d(X, QW, thresholds, btn, type, padding1, padding2, stride1, stride2, N
     return Y
 
 
+def conv2d_launches(X, type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW):
+    """Kernels one Conv2d call with these arguments enqueues: 1 (quantize and convolution in one launch) or 2."""
+    return _lib.tab_conv2d_launches(X.data_ptr(), *(int(v) for v in (type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW)))
+
+
 def static_scratch_bytes():
     """Size of the scratch array built into the library that Conv2dStatic packs the activation into."""
     return _lib.tab_static_scratch_bytes()
@@ -304,7 +337,7 @@ CONV_AUTO, CONV_MATRIX, CONV_POPCOUNT = 0, 1, 2
 
 
 def set_conv_kernel(kernel=CONV_AUTO, tile=-1):
-    """Pick the conv kernel (process-wide): CONV_AUTO, CONV_MATRIX (tile 0..6 or -1) or
+    """Pick the conv kernel (process-wide): CONV_AUTO, CONV_MATRIX (tile 0..9 or -1) or
     CONV_POPCOUNT (tile 0..2 or -1).  Every choice gives bit-identical outputs."""
     _capi.check(_lib, _lib.tab_set_conv_kernel(int(kernel), int(tile)))
 
@@ -313,6 +346,6 @@ def set_conv_kernel(kernel=CONV_AUTO, tile=-1):
 TAB_Quantize = Quantize
 TAB_Conv2d = Conv2d
 
-__all__ = ["Quantize", "QuantizeNCHW", "QuantizeFormat", "Conv2d", "Conv2dStatic", "static_scratch_bytes", "Conv2dPacked", "Conv2dPackedOut", "Threshold", "TAB_Quantize", "TAB_Conv2d", "TabError",
+__all__ = ["Quantize", "QuantizeNCHW", "QuantizeActivation", "conv2d_launches", "QuantizeFormat", "Conv2d", "Conv2dStatic", "static_scratch_bytes", "Conv2dPacked", "Conv2dPackedOut", "Threshold", "TAB_Quantize", "TAB_Conv2d", "TabError",
            "packed_channels", "out_shape", "version", "TNN", "TBN", "BTN", "BNN", "set_conv_kernel",
            "CONV_AUTO", "CONV_MATRIX", "CONV_POPCOUNT"]

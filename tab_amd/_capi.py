@@ -25,6 +25,7 @@ SIGNATURES = {
     "tab_threshold": (_int, [_vp, _int, ctypes.c_long, ctypes.c_float, _vp, _vp, _sz, _vp]),
     "tab_conv2d_workspace_bytes": (_sz, [_int] * 5),
     "tab_conv2d": (_int, [_vp] * 4 + [_int] * 12 + [_vp, _vp, _sz, _vp]),
+    "tab_conv2d_launches": (_int, [_vp] + [_int] * 12),
     "tab_static_scratch_bytes": (_sz, []),
     "tab_conv2d_static": (_int, [_vp] * 4 + [_int] * 12 + [_vp, _vp]),
     "tab_conv2d_packed": (_int, [_vp] * 3 + [_int] * 12 + [_vp, _vp]),

@@ -11,7 +11,9 @@ SOURCES = ["tab_capi.hip", "tab_conv.hip", "tab_conv_mfma_tnn.hip", "tab_conv_mf
 OBJ_DIR = os.path.join(LIB_DIR, "obj")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -packed-fp32-ops: keep the compiler from forming packed-FP32 VALU ops from float code.
-HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-result",
+# -Werror=pass-failed: a kernel whose amdgpu_waves_per_eu request the compiler cannot meet fails the build, so that the
+# residency the shape model counts on is the residency that was compiled.
+HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-result", "-Werror=pass-failed",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 

@@ -95,6 +95,16 @@ const char *tab_version(void) { return "tab_amd 0.1 gfx950"; }
 /* Test hook, absent from include/tab_amd.h: the kernels' multiply-shift division evaluated on the host (x < 2^31, 1 <= d < 2^31). */
 uint32_t tab_internal_div32(uint32_t x, uint32_t d) { return tab::div32(x, tab::make_div32(d)); }
 
+/* Test hook, absent from include/tab_amd.h: the matrix-core workgroup shape the library would pick for an M x KN output with
+ * G = taps * PC words of K (packed: thresholded output), and the duration in microseconds its model predicts for it. */
+int tab_internal_conv_shape(int type, int M, int KN, int G, int PC, int packed, float *cost_us)
+{
+    tab::ConvArgs a = {};
+    a.M = M; a.KN = KN; a.G = G; a.PC = PC;
+    a.qy = packed ? reinterpret_cast<uint32_t *>(&a) : nullptr;  // only tested against null
+    return tab::conv_mfma_shape(type, a, cost_us);
+}
+
 int tab_set_conv_kernel(int kernel, int tile)
 {
     static const int popcount_tm[4] = {7, 8, 4, 2};  // 7: the popcount kernel's own choice
@@ -118,7 +128,7 @@ int tab_quantize(const float *dev_X, const float *dev_ths, int bitwidth, int N, 
 {
     if (bitwidth != 1 && bitwidth != 2) return fail(TAB_ERR_BAD_ARGUMENT, "bitwidth must be 1 or 2, got %d", bitwidth);
     if (N < 1 || H < 1 || W < 1 || C < 1) return fail(TAB_ERR_BAD_ARGUMENT, "N, H, W, C must be positive");
-    if (!dev_X || !dev_ths || !dev_QX || !dev_BTN) return fail(TAB_ERR_BAD_ARGUMENT, "null device pointer");
+    if (!dev_X || !dev_ths || !dev_QX) return fail(TAB_ERR_BAD_ARGUMENT, "null device pointer");  // dev_BTN may be NULL
     if (((uintptr_t)dev_X % 4) || ((uintptr_t)dev_QX % (8 * bitwidth)))
         return fail(TAB_ERR_BAD_ARGUMENT, "X must be aligned to its floats and QX to a whole packed element (%d bytes)", 8 * bitwidth);
     hipError_t e = tab::launch_quantize(dev_X, dev_ths, bitwidth, (long)H * W, N, C,
@@ -133,7 +143,7 @@ int tab_quantize_nchw(const float *dev_X, const float *dev_ths, int bitwidth, in
 {
     if (bitwidth != 1 && bitwidth != 2) return fail(TAB_ERR_BAD_ARGUMENT, "bitwidth must be 1 or 2, got %d", bitwidth);
     if (N < 1 || H < 1 || W < 1 || C < 1) return fail(TAB_ERR_BAD_ARGUMENT, "N, C, H, W must be positive");
-    if (!dev_X || !dev_ths || !dev_QX || !dev_BTN) return fail(TAB_ERR_BAD_ARGUMENT, "null device pointer");
+    if (!dev_X || !dev_ths || !dev_QX) return fail(TAB_ERR_BAD_ARGUMENT, "null device pointer");  // dev_BTN may be NULL
     if (((uintptr_t)dev_X % 4) || ((uintptr_t)dev_QX % (8 * bitwidth)))
         return fail(TAB_ERR_BAD_ARGUMENT, "X must be aligned to its floats and QX to a whole packed element (%d bytes)", 8 * bitwidth);
     if (((long)N * H * W + 255) / 256 * tab_packed_channels(C) > kMaxIndex)
@@ -365,6 +375,14 @@ int tab_conv2d(const float *dev_X, const int64_t *dev_QW, const float *dev_ths,
 {
     return conv_from_floats(dev_X, dev_QW, dev_ths, dev_btn, type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW,
                             dev_Y, workspace, workspace_bytes, false, stream);
+}
+
+int tab_conv2d_launches(const float *dev_X, int type, int padding1, int padding2, int stride1, int stride2, int N, int H, int W,
+                        int C, int KN, int KH, int KW)
+{
+    ConvShape s;
+    if (check_conv(type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW, &s) != TAB_OK) return 0;
+    return !tab::conv_kernel_forced() && tab::conv1x1_fused_supported(type, dev_X, C, KH, KW, padding1, padding2, s.M, KN) ? 1 : 2;
 }
 
 size_t tab_static_scratch_bytes(void) { return TAB_STATIC_SCRATCH_BYTES; }

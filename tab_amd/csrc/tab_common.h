@@ -78,6 +78,9 @@ struct ConvArgs {
     Div32 div_pixels, div_ow;  // by OH*OW and OW: an output row's image and line
 };
 
+// Compute units of the current device (256 on MI355X), looked up once; 256 if the lookup fails.
+int device_compute_units();
+
 // Launchers (tab_conv.hip / tab_quantize.hip); they enqueue on `stream` and return the
 // launch status.
 hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream);
@@ -85,7 +88,7 @@ hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream);
 // short enough for its fp32 accumulators to hold every partial sum exactly.
 bool conv_mfma_exact(const ConvArgs &args);
 bool conv_mfma_exact_levels(const ConvArgs &args);  // the same for type 4, whose products reach 9
-int conv_mfma_shape(int type, const ConvArgs &args);
+int conv_mfma_shape(int type, const ConvArgs &args, float *cost_us = nullptr);
 hipError_t launch_conv_mfma(int type, const ConvArgs &args, int shape, hipStream_t stream);
 hipError_t launch_conv_mfma_tnn(const ConvArgs &args, int shape, hipStream_t stream);
 hipError_t launch_conv_mfma_tbn(const ConvArgs &args, int shape, hipStream_t stream);

@@ -342,6 +342,24 @@ void force_conv_tile(int tm, int ng)
     g_forced_kernel.store(tm == 0 ? 0 : ((tm << 8) | ((ng + 1) & 0xff)), std::memory_order_relaxed);
 }
 
+int device_compute_units()
+{
+    static std::atomic<int> cached{0};
+    int cus = cached.load(std::memory_order_relaxed);
+    if (cus == 0) {
+        int device = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&device) == hipSuccess && hipGetDeviceProperties(&prop, device) == hipSuccess && prop.multiProcessorCount > 0) {
+            cus = prop.multiProcessorCount;
+        } else {
+            (void)hipGetLastError();
+            cus = 256;
+        }
+        cached.store(cus, std::memory_order_relaxed);
+    }
+    return cus;
+}
+
 bool conv_kernel_forced() { return g_forced_kernel.load(std::memory_order_relaxed) != 0; }
 
 // fp32 accumulators hold integers up to 2^24 exactly; a product is at most 1 (9 for the 2-bit levels of
@@ -364,15 +382,16 @@ hipError_t launch_conv_mfma(int type, const ConvArgs &args, int shape, hipStream
 }
 
 // Workgroup tile of the matrix-core kernel: the shape with the lowest predicted duration under a cost model fitted to
-// the measured duration of every shape on 280 (type, layer) cases (tab_conv_shape_model.h: the ResNet-18 layers at
+// the measured duration of every shape on some 290 (type, layer) cases (tab_conv_shape_model.h: the ResNet-18 layers at
 // N = 16 / 64 / 256, the VGG stack, the 28x28 sweep and layers of other geometries).  What the model's features say:
-// the busiest of the 256 CUs decides (ceil(tiles / 256) tiles of a shape land on it, and it is refilled when it holds
-// no more), K scales the loop, the size of Y the epilogue (with a price of its own where K is at most nine words and
-// the launch is little but epilogue), and a launch smaller than the chip is as long as one tile.
-// A shape whose filter tile is at least twice the 64-rounded filter count is no candidate.  Regret of the choice
-// against the best measured shape: 1.0 % over the fitted cases, 1.4 % with each layer set held out of the fit in turn
-// (the thresholds this replaces: 2.8 % on their measurements, 5.5 % on the geometries they were not made from).
-int conv_mfma_shape(int conv_type, const ConvArgs &a)
+// the busiest CU decides (ceil(tiles / CUs) tiles of a shape land on it, and it is refilled when it holds no more), K
+// scales the loop, the size of Y the epilogue (with a price of its own where K is at most nine words and the launch is
+// little but epilogue), and a launch smaller than the chip is as long as one tile.  Features and coefficients are all
+// non-negative, so a prediction is positive and monotone in K, tiles and Y for any geometry; on top of that no prediction
+// is taken below what the matrix cores of the busiest CU need at their peak rate plus a launch.
+// A shape whose filter tile is at least twice the 64-rounded filter count is no candidate.
+// cost_us (optional): the predicted duration of the chosen shape.
+int conv_mfma_shape(int conv_type, const ConvArgs &a, float *cost_us)
 {
     // the CPU-only types follow the type with the same planes: 4 like TNN, 5 like BNN
     const int type = conv_type == 4 ? 0 : (conv_type == 5 ? 3 : conv_type);
@@ -380,30 +399,40 @@ int conv_mfma_shape(int conv_type, const ConvArgs &a)
     // thresholds a pixel's filters inside a lane, runs 1.4-2x faster than the tiled shapes once the launch is a few
     // rounds of waves (N=256 56x56x64->64 3x3: 24 against 38 us) and level with them on small ones; with fp32 output
     // both are bound by writing Y and measure within 5 % of each other, so the tiled shapes keep those launches
-    if (conv_type <= 3 && a.G <= 9 && a.qy != nullptr && (a.M >= 65536 || a.G <= 2)) return 7;
+    if (conv_type <= 3 && a.G <= 9 && a.qy != nullptr && (a.M >= 65536 || a.G <= 2)) {
+        if (cost_us) *cost_us = 0.f;
+        return 7;
+    }
     const long kn64 = ((long)a.KN + 63) / 64 * 64;
+    const long cus = device_compute_units();
     // (packed output ranks the shapes as fp32 output does: the model's terms in Y also stand for what grows with M * KN)
     const float y_mb = (float)a.M * (float)a.KN * 4e-6f;
     int best = 2;
     float best_cost = 0.f;
     bool any = false;
-    for (int shape = 0; shape < kConvShapes; shape++) {
-        const int bm = kConvShapeTile[shape][0], bn = kConvShapeTile[shape][1], held = kConvShapeTile[shape][2];
+    for (int i = 0; i < kConvShapes; i++) {
+        const int shape = kConvShapeIds[i];
+        const int bm = kConvShapeTile[i][0], bn = kConvShapeTile[i][1], held = kConvShapeTile[i][2];
         if (bn >= 2 * kn64) continue;
-        if (shape == 3 && a.qy != nullptr) continue;  // the packed epilogues need tiles 64 filters wide
+        if (shape == 3 && a.qy != nullptr) continue;        // the packed epilogues need tiles 64 filters wide
+        if (shape >= 8 && a.PC % 2 != 0) continue;          // the split-K shapes move whole pairs of words inside a tap
         const long tiles = (long)((a.M + bm - 1) / bm) * ((a.KN + bn - 1) / bn);
-        const float n = (float)((tiles + 255) / 256), rounds = (float)(((tiles + 255) / 256 + held - 1) / held);
-        const float busy = tiles >= 256 ? 1.f : (float)tiles / 256.f;
+        const float n = (float)((tiles + cus - 1) / cus), rounds = (float)(((tiles + cus - 1) / cus + held - 1) / held);
+        const float busy = tiles >= cus ? 1.f : (float)tiles / (float)cus;
         const float f[kConvShapeFeatures] = {(float)a.G * n, (float)a.G * rounds, rounds, n, y_mb, y_mb * busy, busy, 1.f,
                                              a.G <= 9 ? y_mb : 0.f};
         float cost = 0.f;
-        for (int i = 0; i < kConvShapeFeatures; i++) cost += kConvShapeCost[type][shape][i] * f[i];
+        for (int k = 0; k < kConvShapeFeatures; k++) cost += kConvShapeCost[type][i][k] * f[k];
+        // the busiest CU's n tiles of (bm/32)(bn/32) MFMA tiles x G words, 32 cycles each on four SIMDs at 2.4 GHz, and a launch
+        const float floor_us = 1.f + n * (float)(bm / 32 * (bn / 32)) * (float)a.G * (32.f / 4.f / 2400.f);
+        if (cost < floor_us) cost = floor_us;
         if (!any || cost < best_cost) {
             any = true;
             best = shape;
             best_cost = cost;
         }
     }
+    if (cost_us) *cost_us = best_cost;
     return best;
 }
 

@@ -481,12 +481,31 @@ long order_workgroups(ConvArgs &a, int tiles_n)
     return by_rows_of_y ? (long)((a.tiles_m + 7) / 8) * 8 * tiles_n : (long)a.tiles_m * tiles_n;
 }
 
-// waves_per_eu: the shapes with four MFMA tiles per wave are capped at 128 registers, i.e. four
-// workgroups per CU (the 128x128 shape otherwise takes 136-152, 64 of them accumulators, and runs
-// three, measured 3-7 % slower); 256-row tiles need the state of more staged rows and get 168
-// (three workgroups), eight tiles per wave 256 (two).
+// LDS of a CU, and the workgroups of four waves (one wave per SIMD each) that a CU holds by it.
+constexpr int kLdsBytesPerCu = 160 * 1024;
+constexpr int waves_by_lds(int lds_bytes) { return lds_bytes <= 0 ? 8 : (kLdsBytesPerCu / lds_bytes < 1 ? 1 : kLdsBytesPerCu / lds_bytes); }
+
+// Waves per SIMD asked of the register allocation.  The shapes with four MFMA tiles per wave are capped at 128
+// registers, i.e. four workgroups per CU (the 128x128 shape otherwise takes 136-152, 64 of them accumulators, and runs
+// three, measured 3-7 % slower); 256-row tiles need the state of more staged rows and get 168 (three workgroups), eight
+// tiles per wave 256 (two).  Never more than the LDS of the workgroup lets a CU hold: a request beyond that only costs
+// registers.
+constexpr int mfma_waves_per_eu(int wm, int tm, int tn, int lds_bytes)
+{
+    const int by_registers = tm * tn > 4 ? 2 : (wm * tm > 4 ? 3 : 4);
+    return waves_by_lds(lds_bytes) < by_registers ? waves_by_lds(lds_bytes) : by_registers;
+}
+template <int TYPE, int WM, int WN, int TM, int TN, int KCH, bool INTAP, int KS>
+constexpr int conv_mfma_lds_bytes()
+{
+    constexpr int BM = 32 * WM * TM, BN = 32 * WN * TN;
+    using Stager = typename std::conditional<INTAP, TapStager<TYPE, BM, BN, INTAP ? KCH : 2>, TileStager<TYPE, BM, BN, KCH>>::type;
+    return 4 * (2 * (Stager::A_DWORDS + Stager::B_DWORDS) + (KS > 1 ? KS * 17 * 64 : 1));
+}
+
 template <int TYPE, int WM, int WN, int TM, int TN, int KCH, bool INTAP, int KS = 1>
-__global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TM * TN > 4 ? 2 : (WM * TM > 4 ? 3 : 4)))) void conv_mfma(const ConvArgs p)
+__global__ __launch_bounds__(kConvThreads)
+__attribute__((amdgpu_waves_per_eu(mfma_waves_per_eu(WM, TM, TN, conv_mfma_lds_bytes<TYPE, WM, WN, TM, TN, KCH, INTAP, KS>())))) void conv_mfma(const ConvArgs p)
 {
     static_assert(WM * WN * KS * 64 == kConvThreads, "four waves");
     static_assert(KCH % KS == 0 && (KS == 1 || (TM == 1 && TN == 1)), "k-split waves share one 32x32 tile");

@@ -46,13 +46,6 @@ __device__ __forceinline__ int run_swizzle(int row)
     return RUN == 4 ? ((row >> 1) + (row >> 3)) & 3 : (RUN == 2 ? ((row >> 2) + (row >> 3)) & 1 : 0);
 }
 
-// Waves per SIMD the register allocation is asked for: four with up to four MFMA tiles a wave (128 registers), three
-// with 256-row tiles (the state of more staged rows), two with eight tiles a wave.
-constexpr int direct_waves_per_eu(int type, int wm, int tm, int tn, int ks)
-{
-    return tm * tn > 4 ? 2 : (wm * tm > 4 && ks == 1 ? 3 : 4);
-}
-
 // LDS dwords one wave deposits per 32x32 tile when KS waves exchange partial sums: 16 accumulator elements a lane as four
 // 16-byte quads, quad q of lane l at dword q * 256 + 4 * l (consecutive lanes 16 bytes apart: conflict-free 16-byte
 // accesses), then one dword a lane for BTN's count of nonzero weight bits.
@@ -69,8 +62,21 @@ constexpr int kSplitRoundTiles = 2;  // tiles a wave deposits per exchange round
 // multiple of the chunk: words past it are fetched as zeros (the BNN bias counts them).
 // ARUN: granules of an activation row that neighbouring lanes fetch (0: the widest the chunk allows); a run must not
 // straddle filter taps, so layers with few words per pixel take a shorter one.
+template <int TYPE, int WM, int WN, int TM, int TN, int KCH, int KS>
+constexpr int conv_mfma_direct_lds_dwords()
+{
+    constexpr int APL = Planes<TYPE>::A, BPL = Planes<TYPE>::B;
+    constexpr int BM = 32 * WM * TM, BN = 32 * WN * TN;
+    constexpr int A_ITEMS = (KCH * APL / 2 * BM + kConvThreads - 1) / kConvThreads, B_ITEMS = (KCH * BPL / 2 * BN + kConvThreads - 1) / kConvThreads;
+    constexpr int buffers = 2 * 4 * (A_ITEMS + B_ITEMS) * kConvThreads;  // two chunks of whole wave instructions
+    // partial sums of the KS wave groups: kSplitRoundTiles tiles per wave and round, then the packed epilogue's 32 dwords a wave
+    constexpr int split = KS > 1 ? (kConvThreads / 64) * (kSplitRoundTiles * kSplitTileDwords + 32) : 0;
+    return buffers > split ? buffers : split;
+}
+
 template <int TYPE, int WM, int WN, int TM, int TN, int KCH, bool PACKED, int KS = 1, int ARUN = 0>
-__global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(direct_waves_per_eu(TYPE, WM, TM, TN, KS)))) void conv_mfma_direct(const ConvArgs p)
+__global__ __launch_bounds__(kConvThreads)
+__attribute__((amdgpu_waves_per_eu(mfma_waves_per_eu(KS > 1 ? 1 : WM, TM, TN, 4 * conv_mfma_direct_lds_dwords<TYPE, WM, WN, TM, TN, KCH, KS>())))) void conv_mfma_direct(const ConvArgs p)
 {
     static_assert(WM * WN * KS * 64 == kConvThreads && KCH % (2 * KS) == 0, "four waves, whole pairs of words per wave group");
     constexpr int PAIRS = KCH / 2;
@@ -84,10 +90,7 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(di
     constexpr int A_RUN = ARUN ? ARUN : granule_run(PA, APL), B_RUN = granule_run(PB, BPL);
     static_assert(BM % 64 == 0 && BN % 64 == 0, "one wave instruction moves 64 / RUN rows of one run");
     static_assert(PA % A_RUN == 0, "whole runs");
-    // partial sums of the KS wave groups: kSplitRoundTiles tiles per wave and round, then the packed epilogue's 32 dwords a wave
-    constexpr int SPLIT_DWORDS = KS > 1 ? (kConvThreads / 64) * (kSplitRoundTiles * kSplitTileDwords + 32) : 0;
-
-    __shared__ __attribute__((aligned(16))) uint32_t lds[2 * BUF_DWORDS > SPLIT_DWORDS ? 2 * BUF_DWORDS : SPLIT_DWORDS];
+    __shared__ __attribute__((aligned(16))) uint32_t lds[conv_mfma_direct_lds_dwords<TYPE, WM, WN, TM, TN, KCH, KS>()];
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;

@@ -25,6 +25,8 @@
 #pragma once
 #include "tab_conv_mfma.h"
 
+#include <atomic>
+
 namespace tab {
 namespace {
 
@@ -328,22 +330,21 @@ hipError_t launch_mfma_regs_tile(ConvArgs a, hipStream_t stream)
 {
     const int tiles_n = (a.KN + 32 * TN - 1) / (32 * TN);
     if (tiles_n > 65535) return hipErrorInvalidValue;
-    static int per_cu = 0;  // resident workgroups per CU
-    static int cus = 0;
-    if (per_cu == 0) {
-        int blocks = 0, device = 0;
-        hipDeviceProp_t prop;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, conv_mfma_regs<TYPE, G, TN, OUT>, kConvThreads, 0) != hipSuccess ||
-            hipGetDevice(&device) != hipSuccess || hipGetDeviceProperties(&prop, device) != hipSuccess) {
+    // workgroups the chip holds at once (resident workgroups per CU x CUs), looked up on the first launch and kept in
+    // one atomic word: threads that race here compute the same value, and a reader sees either 0 or all of it
+    static std::atomic<int> resident{0};
+    int held = resident.load(std::memory_order_relaxed);
+    if (held == 0) {
+        int blocks = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, conv_mfma_regs<TYPE, G, TN, OUT>, kConvThreads, 0) != hipSuccess) {
             (void)hipGetLastError();
             blocks = 2;
-            prop.multiProcessorCount = 256;
         }
-        cus = prop.multiProcessorCount;
-        per_cu = blocks < 1 ? 1 : blocks;
+        held = device_compute_units() * (blocks < 1 ? 1 : blocks);
+        resident.store(held, std::memory_order_relaxed);
     }
     const int tiles = (a.M + 31) / 32;
-    const int cap = (cus * per_cu + tiles_n - 1) / tiles_n;
+    const int cap = (held + tiles_n - 1) / tiles_n;
     a.kcw = G;
     a.nchunks = 1;
     conv_mfma_regs<TYPE, G, TN, OUT><<<dim3(regs_grid_x(tiles, cap < 1 ? 1 : cap), (unsigned)tiles_n), dim3(kConvThreads), 0, stream>>>(a);

@@ -1,51 +1,64 @@
-// Written by tab_amd/tuning/fit_conv_shape_model.py from tab_amd/tuning/conv_shape_timings.txt: do not edit.
-// Cost model of the matrix-core workgroup shapes: predicted duration (us) = kConvShapeCost[type][shape] . f,
-// f = {G*n, G*rounds, rounds, n, Y, Y*busy, busy, 1, Y*[G <= 9]} (tiles on the busiest CU, refills of that CU, megabytes
-// of Y, share of the CUs with work).  Regret of the choice against the best measured shape over the
-// 280 fitted cases: 1.02%; with each layer set held out of the fit in turn: 1.38%.
+// Written by tab_amd/tuning/fit_conv_shape_model.py from tab_amd/tuning/conv_shape_training_timings.txt: do not edit.
+// Fitted 2026-11-25 on the kernels of commit 94eeb72 (and the working tree on top of it).
+// Cost model of the matrix-core workgroup shapes: predicted duration (us) = kConvShapeCost[type][i] . f for the shape
+// kConvShapeIds[i], f = {G*n, G*rounds, rounds, n, Y, Y*busy, busy, 1, Y*[G <= 9]} (n = tiles on the busiest CU,
+// rounds = refills of that CU, Y = megabytes of output, busy = share of the CUs with work).  Non-negative least squares:
+// every feature and every coefficient is >= 0, so a prediction is positive and monotone for any geometry.  Regret of the
+// choice against the best measured shape over the 280 fitted cases: 1.19%; with each layer set held out of
+// the fit in turn: 1.65%.
 #pragma once
 
 namespace tab {
 
-constexpr int kConvShapes = 7, kConvShapeFeatures = 9;
-// rows x filters of the workgroup tile and workgroups a CU holds, per shape
-constexpr int kConvShapeTile[kConvShapes][3] = {{128, 128, 4}, {128, 64, 4}, {64, 64, 4}, {32, 32, 8}, {256, 64, 3}, {256, 128, 2}, {128, 256, 2}};
+constexpr int kConvShapes = 9, kConvShapeFeatures = 9;
+// the shape ids tab_set_conv_kernel(TAB_CONV_MATRIX, id) takes, in the order of the tables below
+constexpr int kConvShapeIds[kConvShapes] = {0, 1, 2, 3, 4, 5, 6, 8, 9};
+// rows x filters of the workgroup tile and workgroups a CU holds (compiled occupancy), per shape
+constexpr int kConvShapeTile[kConvShapes][3] = {{128, 128, 4}, {128, 64, 6}, {64, 64, 8}, {32, 32, 4}, {256, 64, 4}, {256, 128, 2}, {128, 256, 2}, {64, 64, 4}, {128, 128, 2}};
 constexpr float kConvShapeCost[4][kConvShapes][kConvShapeFeatures] = {
     {
-        {0.101736f, 0.0783438f, -0.68712f, 1.01087f, 0.435055f, -0.425774f, 1.72623f, 1.87135f, 0.0700297f},
-        {0.0592816f, 0.0761902f, 0.252233f, 0.308101f, -0.115512f, 0.12106f, 2.01476f, 2.03173f, 0.0508505f},
-        {0.0402916f, 0.0367362f, -0.7858f, 0.989465f, 0.708673f, -0.805977f, 1.77938f, 1.24847f, 0.0211692f},
-        {0.0271031f, -0.00476068f, -0.485913f, 0.409288f, 0.00600619f, 0.00600619f, 1.41759f, 1.41759f, -0.0835859f},
-        {0.0921229f, 0.115016f, 0.521055f, -0.0407646f, 0.324878f, -0.282047f, 2.18356f, 2.08351f, 0.0649364f},
-        {0.164875f, 0.0994395f, 0.386205f, 1.46624f, 0.354393f, -0.300854f, 1.30748f, 2.12057f, 0.043873f},
-        {0.119585f, 0.131126f, 0.768355f, 0.998577f, 0.0922746f, -0.00369637f, 1.24234f, 2.35936f, 0.0122326f},
+        {0.09622f, 0.0755577f, 0.0f, 0.0f, 0.0606748f, 0.0f, 1.7507f, 3.14281f, 0.0612442f},
+        {0.0671462f, 0.0682265f, 0.0f, 0.0f, 0.0f, 0.0534564f, 1.63501f, 2.45946f, 0.0502946f},
+        {0.0451608f, 0.0317093f, 0.0f, 0.42626f, 0.0f, 0.0f, 0.784499f, 2.03594f, 0.0142967f},
+        {0.0269856f, 0.0f, 0.0716856f, 0.263235f, 0.0f, 0.0f, 2.58355f, 0.0f, 0.0f},
+        {0.100423f, 0.10475f, 0.0f, 0.0f, 0.0485751f, 0.0f, 2.34609f, 3.21895f, 0.0618952f},
+        {0.150327f, 0.110511f, 0.0f, 0.0f, 0.0932148f, 0.0f, 1.78975f, 4.71658f, 0.0422527f},
+        {0.128618f, 0.118425f, 0.0f, 0.0f, 0.0723173f, 0.0463867f, 0.743713f, 4.19554f, 0.0173782f},
+        {0.0251956f, 0.0396773f, 0.0f, 0.670934f, 0.0254314f, 0.0f, 0.734947f, 3.29611f, 0.0f},
+        {0.0628066f, 0.0892484f, 0.826519f, 0.0390676f, 0.112093f, 0.0f, 0.0317503f, 4.3067f, 0.0159801f},
     },
     {
-        {0.0894807f, 0.0732002f, -0.601899f, 0.868973f, 0.394591f, -0.377651f, 1.66654f, 1.8411f, 0.0718983f},
-        {0.050817f, 0.0718902f, 0.0412541f, 0.421336f, -0.129168f, 0.128296f, 1.71719f, 2.09767f, 0.0543004f},
-        {0.0329458f, 0.0370061f, -0.755188f, 1.05107f, 0.525997f, -0.642743f, 1.61356f, 1.31199f, 0.0199901f},
-        {0.0209509f, 0.00168176f, -0.594492f, 0.0276148f, 0.146077f, 0.146077f, 1.54632f, 1.54632f, -0.0092348f},
-        {0.0798248f, 0.116957f, 0.260442f, 0.0704327f, 0.311755f, -0.2556f, 2.19701f, 2.05316f, 0.0538066f},
-        {0.163936f, 0.0738744f, 0.158364f, 1.39251f, 0.384372f, -0.330225f, 1.15497f, 2.11986f, 0.0436855f},
-        {0.117375f, 0.0788366f, 0.64263f, 0.913006f, 0.094183f, 0.00239735f, 1.06351f, 2.3725f, 0.00715049f},
+        {0.0865426f, 0.0693587f, 0.0f, 0.0f, 0.0579624f, 0.0f, 1.82022f, 2.9411f, 0.0648396f},
+        {0.0586298f, 0.0641694f, 0.0f, 0.209004f, 0.0f, 0.0279674f, 1.52226f, 2.17486f, 0.0554612f},
+        {0.0383737f, 0.0306837f, 0.0f, 0.412396f, 0.0f, 0.0f, 0.885265f, 1.92272f, 0.0116986f},
+        {0.0210085f, 0.00123058f, 0.326048f, 0.171836f, 0.0f, 0.0f, 2.45928f, 0.0f, 0.0f},
+        {0.0943118f, 0.0969396f, 0.0f, 0.0f, 0.0546803f, 0.0f, 2.36483f, 2.9726f, 0.0584947f},
+        {0.13924f, 0.0996686f, 0.0f, 0.0f, 0.0861756f, 0.0f, 2.11001f, 4.45851f, 0.0409859f},
+        {0.121266f, 0.0798943f, 0.0f, 0.0f, 0.0885932f, 0.0317639f, 0.564441f, 3.91746f, 0.0156865f},
+        {0.022049f, 0.0348356f, 0.0f, 0.768156f, 0.0f, 0.0f, 0.620039f, 3.04518f, 0.0f},
+        {0.0613883f, 0.0738368f, 1.12291f, 0.0f, 0.0950171f, 0.0f, 0.305162f, 3.77746f, 0.0184637f},
     },
     {
-        {0.0963754f, 0.0647816f, -0.520498f, 0.860092f, 0.411138f, -0.399735f, 1.60518f, 1.85106f, 0.0777457f},
-        {0.0613087f, 0.0592151f, 0.290415f, 0.311998f, -0.11528f, 0.102375f, 1.94103f, 1.90556f, 0.0730051f},
-        {0.0371194f, 0.0300203f, -0.651056f, 0.991019f, 0.502189f, -0.63366f, 1.7372f, 1.26138f, 0.0403837f},
-        {0.0218465f, 0.00141591f, -0.499721f, -0.0403127f, 0.177208f, 0.177208f, 1.59077f, 1.59077f, 0.0216665f},
-        {0.0977166f, 0.0733417f, 0.354856f, -0.229322f, 0.33864f, -0.301939f, 2.18212f, 2.08557f, 0.0893625f},
-        {0.175103f, 0.0171519f, 0.121538f, 1.38135f, 0.377705f, -0.327717f, 0.982463f, 1.9917f, 0.0553879f},
-        {0.133522f, 0.0788339f, 0.683095f, 1.1073f, 0.121279f, -0.0289249f, 0.95748f, 2.35545f, 0.00371973f},
+        {0.0921608f, 0.0695768f, 0.0f, 0.0f, 0.0494465f, 0.0f, 1.69354f, 3.09981f, 0.0724312f},
+        {0.0669284f, 0.0552975f, 0.0f, 0.0f, 0.0f, 0.0334096f, 1.58694f, 2.38494f, 0.0745116f},
+        {0.0416222f, 0.0198294f, 0.0f, 0.322649f, 0.0f, 0.0f, 0.74886f, 2.16381f, 0.0347851f},
+        {0.0201173f, 0.00501934f, 0.423686f, 0.190298f, 0.0f, 0.0f, 2.50451f, 0.0f, 0.0f},
+        {0.101425f, 0.0651953f, 0.174489f, 0.0f, 0.0228169f, 0.0f, 2.59556f, 2.74479f, 0.0876685f},
+        {0.152702f, 0.0380489f, 0.0f, 0.0f, 0.083621f, 0.0f, 1.93433f, 4.31916f, 0.0504919f},
+        {0.138187f, 0.0742667f, 0.0f, 0.0f, 0.0964049f, 0.0304895f, 0.290869f, 4.27502f, 0.00752971f},
+        {0.0234524f, 0.0278454f, 0.0f, 0.699996f, 0.0246471f, 0.0f, 0.61602f, 3.03661f, 0.00496521f},
+        {0.0751333f, 0.0522657f, 0.737833f, 0.0181711f, 0.116729f, 0.0f, 0.0f, 4.44661f, 0.00639848f},
     },
     {
-        {0.0757081f, 0.0549324f, -0.677878f, 0.929788f, 0.437617f, -0.410386f, 1.56424f, 1.80487f, 0.0647654f},
-        {0.0462825f, 0.0620089f, 0.212905f, 0.301511f, -0.175386f, 0.161165f, 1.70891f, 2.00495f, 0.0833854f},
-        {0.0303778f, 0.023491f, -0.742222f, 1.10325f, 0.439588f, -0.597834f, 1.61526f, 1.36647f, 0.0442665f},
-        {0.0149201f, 0.00728321f, -0.466189f, 0.0621023f, 0.124811f, 0.124811f, 1.5064f, 1.5064f, -0.0374734f},
-        {0.0793136f, 0.0680044f, 0.126478f, -0.259799f, 0.373458f, -0.315692f, 2.0126f, 2.17313f, 0.0813827f},
-        {0.147704f, 0.0381786f, 0.0763775f, 1.30757f, 0.375339f, -0.320703f, 0.911149f, 1.87217f, 0.0547583f},
-        {0.115613f, 0.0552379f, 0.645267f, 0.818287f, 0.123423f, -0.0292234f, 0.923288f, 2.21852f, 0.0122594f},
+        {0.070951f, 0.0583979f, 0.0f, 0.0f, 0.07163f, 0.0f, 1.72993f, 2.88768f, 0.0573304f},
+        {0.051832f, 0.0574573f, 0.0f, 0.186692f, 0.0f, 0.00781961f, 1.67776f, 1.99304f, 0.082882f},
+        {0.0334607f, 0.0209968f, 0.0f, 0.27473f, 0.0f, 0.0f, 0.746789f, 2.1151f, 0.0449228f},
+        {0.0165723f, 0.000672762f, 0.409753f, 0.120531f, 0.0f, 0.0f, 2.55998f, 0.0f, 0.0f},
+        {0.0815124f, 0.060848f, 0.0f, 0.0f, 0.0399928f, 0.0f, 2.50892f, 2.79836f, 0.0794404f},
+        {0.132555f, 0.0385214f, 0.0f, 0.0f, 0.0873704f, 0.0f, 1.8309f, 4.08767f, 0.049155f},
+        {0.123896f, 0.040661f, 0.0f, 0.0f, 0.0945826f, 0.0255268f, 0.42759f, 3.8027f, 0.0161334f},
+        {0.0182987f, 0.0251055f, 0.0f, 0.701043f, 0.0083251f, 0.0f, 0.680731f, 2.86485f, 0.00394225f},
+        {0.0638827f, 0.0401316f, 1.02065f, 0.0f, 0.103476f, 0.0f, 0.113542f, 3.80058f, 0.0134501f},
     },
 };
 

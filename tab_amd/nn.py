@@ -8,7 +8,7 @@ Inference only (the operators have no backward).
 import torch
 from torch import nn
 
-from . import (BNN, BTN, TBN, TNN, Conv2d, Conv2dPacked, Conv2dPackedOut, Quantize, QuantizeNCHW, Threshold,
+from . import (BNN, BTN, TBN, TNN, Conv2d, Conv2dPacked, Conv2dPackedOut, Quantize, QuantizeActivation, Threshold,
                out_shape)
 
 _ACT_BITS = {TNN: 2, TBN: 2, BTN: 1, BNN: 1}
@@ -68,7 +68,7 @@ class TABConv2d(nn.Module):
         (KH, KW), (s1, s2), (p1, p2) = self.kernel_size, self.stride, self.padding
         if nchw:
             # quantized straight from NCHW (no transposed fp32 copy), then the packed entry point
-            QX, _ = QuantizeNCHW(x, ths, abits, N, C, H, W)
+            QX = QuantizeActivation(x, ths, abits, N, H, W, C, nchw=True)  # no BTN vector: nobody reads an activation's
             y = Conv2dPacked(QX, self.QW, self.BTN_W, self.conv_type, p1, p2, s1, s2, N, H, W, C,
                              self.out_channels, KH, KW)
         else:
@@ -145,7 +145,7 @@ class TABPackedChain(nn.Module):
         x = x.to(torch.float32).contiguous()
         bits = _ACT_BITS[first.conv_type]
         ths = Threshold(x, N, first.act_scale) if bits == 2 else torch.zeros(N, dtype=torch.float32, device=x.device)
-        q, _ = QuantizeNCHW(x, ths, bits, N, C, H, W) if nchw else Quantize(x, ths, bits, N, H, W, C)
+        q = QuantizeActivation(x, ths, bits, N, H, W, C, nchw=nchw)
         for i, layer in enumerate(self.layers):
             (KH, KW), (s1, s2), (p1, p2) = layer.kernel_size, layer.stride, layer.padding
             args = (layer.conv_type, p1, p2, s1, s2, N, H, W, layer.in_channels, layer.out_channels, KH, KW)

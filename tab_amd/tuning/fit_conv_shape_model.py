@@ -1,6 +1,8 @@
 """Fits the cost model conv_mfma_shape() chooses the workgroup shape with and writes tab_amd/csrc/tab_conv_shape_model.h.
 
-Input: conv_shape_timings.txt (collect_conv_shape_timings.py): per (type, layer) the duration of every shape.
+Input: conv_shape_training_timings.txt, the model's training data: per (type, layer) the measured duration in microseconds of
+every shape on one MI355X (median of three rounds taken round-robin over the shapes, clock warmed; conv kernel alone,
+tab_set_conv_kernel(TAB_CONV_MATRIX, shape)).
 Model, per (type, shape): duration ~ c . f with the features
     f = [G*n, G*rounds, rounds, n, Y, Y*busy, busy, 1, Y*[G <= 9]]
     tiles  = ceil(M / BM) * ceil(KN / BN)            workgroups of the launch
@@ -9,8 +11,11 @@ Model, per (type, shape): duration ~ c . f with the features
     busy   = min(1, tiles / 256)                     share of the CUs that have work at all
     G      = KH*KW*PC words of K, Y = 4*M*KN bytes / 1e6; the last feature gives the layers whose loop is a handful of
              MFMAs (C = 64 with 3x3, 1x1) their own price per byte of Y: their launches are the epilogue
-fitted by least squares on relative error (ridge 1e-2; the N=16 set weighted threefold).  A shape whose filter tile is at least twice the (64-rounded)
-filter count is not a candidate.  The script prints the regret of the model's choice against the best measured shape:
+fitted by NON-NEGATIVE least squares on relative error (the N=16 set weighted threefold): every feature is non-negative and
+so is every coefficient, hence a predicted duration is positive and grows with K, with the tiles on the busiest CU and
+with Y for every geometry, inside the fitted range or far outside it (an unconstrained fit had coefficients of both signs,
+whose predictions can cross or go negative where nothing was measured).  A shape whose filter tile is at least twice the
+(64-rounded) filter count is not a candidate.  The script prints the regret of the model's choice against the best measured shape:
 fitted on everything, and with each set held out in turn.
 
     python tab_amd/tuning/fit_conv_shape_model.py        # needs numpy only"""
@@ -21,7 +26,11 @@ import re
 import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SHAPES = {0: (128, 128, 4), 1: (128, 64, 4), 2: (64, 64, 4), 3: (32, 32, 8), 4: (256, 64, 3), 5: (256, 128, 2), 6: (128, 256, 2)}
+# shape id -> rows x filters of the workgroup tile, workgroups a CU holds (the occupancy the compiler reports for the
+# shape's kernels with four-word chunks: registers, or LDS where that is the tighter limit)
+SHAPES = {0: (128, 128, 4), 1: (128, 64, 6), 2: (64, 64, 8), 3: (32, 32, 4), 4: (256, 64, 4), 5: (256, 128, 2), 6: (128, 256, 2),
+          8: (64, 64, 4), 9: (128, 128, 2)}
+IDS = sorted(SHAPES)
 NFEAT = 9
 
 
@@ -37,12 +46,14 @@ def parse(path):
         t, N, H, W, C, KN, kh, kw, p1, p2, s1, s2 = map(int, m.groups()[:12])
         OH, OW = (H + 2 * p1 - kh + 1) // s1, (W + 2 * p2 - kw + 1) // s2  # TAB_GEMM.cu:354-357
         times = {int(a.split(":")[0]): float(a.split(":")[1]) for a in m.group(13).split()}
-        rows.append(dict(set=which, type=t, M=N * OH * OW, KN=KN, G=kh * kw * ((C + 63) // 64), times=times, name=line.split()[2]))
+        rows.append(dict(set=which, type=t, M=N * OH * OW, KN=KN, G=kh * kw * ((C + 63) // 64), PC=(C + 63) // 64, times=times,
+                         name=line.split()[2]))
     return rows
 
 
 def eligible(r, s):
-    return SHAPES[s][1] < 2 * (-(-r["KN"] // 64) * 64) and s in r["times"]
+    # (the split-K shapes need an even number of words per pixel; otherwise they run as shapes 2 and 0)
+    return SHAPES[s][1] < 2 * (-(-r["KN"] // 64) * 64) and s in r["times"] and not (s >= 8 and r["PC"] % 2)
 
 
 def features(r, s):
@@ -55,7 +66,9 @@ def features(r, s):
     return [r["G"] * n, r["G"] * rounds, rounds, n, Y, Y * busy, busy, 1.0, Y if r["G"] <= 9 else 0.0]
 
 
-def fit(rows, ridge=1e-2):
+def fit(rows):
+    from scipy.optimize import nnls
+
     coef = {}
     for s in SHAPES:
         for t in range(4):
@@ -63,8 +76,7 @@ def fit(rows, ridge=1e-2):
             y = np.array([r["times"][s] for r in rows if r["type"] == t and eligible(r, s)])
             w = 1.0 / np.maximum(y, 1.0)  # relative error; the latency-bound N=16 set, the benchmark's headline, counts threefold
             w = w * np.array([3.0 if r["set"] == "rn16" else 1.0 for r in rows if r["type"] == t and eligible(r, s)])
-            A, b = X * w[:, None], y * w
-            coef[(t, s)] = np.linalg.solve(A.T @ A + ridge * np.eye(NFEAT), A.T @ b)
+            coef[(t, s)] = nnls(X * w[:, None], y * w)[0]
     return coef
 
 
@@ -85,7 +97,7 @@ def regret(rows, coef):
 
 
 def main():
-    rows = parse(os.path.join(HERE, "conv_shape_timings.txt"))
+    rows = parse(os.path.join(HERE, "conv_shape_training_timings.txt"))
     coef = fit(rows)
     total, per = regret(rows, coef)
     sets = sorted(per)
@@ -102,21 +114,30 @@ def main():
     print(f"{len(rows)} cases; regret of the model's choice, fitted on all: {total:.2%} ({', '.join(f'{k} {v:.1%}' for k, v in sorted(per.items()))})")
     print(f"each set held out of the fit in turn: {held_chosen / held_best - 1:.2%} ({', '.join(f'{k} {v:.1%}' for k, v in sorted(held.items()))})")
     out = os.path.join(os.path.dirname(HERE), "csrc", "tab_conv_shape_model.h")
+    import datetime
+    import subprocess
+
+    commit = subprocess.run(["git", "-C", HERE, "rev-parse", "--short", "HEAD"], stdout=subprocess.PIPE, text=True).stdout.strip() or "unknown"
     with open(out, "w") as f:
-        f.write("// Written by tab_amd/tuning/fit_conv_shape_model.py from tab_amd/tuning/conv_shape_timings.txt: do not edit.\n")
-        f.write("// Cost model of the matrix-core workgroup shapes: predicted duration (us) = kConvShapeCost[type][shape] . f,\n")
-        f.write("// f = {G*n, G*rounds, rounds, n, Y, Y*busy, busy, 1, Y*[G <= 9]} (tiles on the busiest CU, refills of that CU, megabytes\n")
-        f.write("// of Y, share of the CUs with work).  Regret of the choice against the best measured shape over the\n")
-        f.write(f"// {len(rows)} fitted cases: {total:.2%}; with each layer set held out of the fit in turn: {held_chosen / held_best - 1:.2%}.\n")
+        f.write("// Written by tab_amd/tuning/fit_conv_shape_model.py from tab_amd/tuning/conv_shape_training_timings.txt: do not edit.\n")
+        f.write(f"// Fitted {datetime.date.today().isoformat()} on the kernels of commit {commit} (and the working tree on top of it).\n")
+        f.write("// Cost model of the matrix-core workgroup shapes: predicted duration (us) = kConvShapeCost[type][i] . f for the shape\n")
+        f.write("// kConvShapeIds[i], f = {G*n, G*rounds, rounds, n, Y, Y*busy, busy, 1, Y*[G <= 9]} (n = tiles on the busiest CU,\n")
+        f.write("// rounds = refills of that CU, Y = megabytes of output, busy = share of the CUs with work).  Non-negative least squares:\n")
+        f.write("// every feature and every coefficient is >= 0, so a prediction is positive and monotone for any geometry.  Regret of the\n")
+        f.write(f"// choice against the best measured shape over the {len(rows)} fitted cases: {total:.2%}; with each layer set held out of\n")
+        f.write(f"// the fit in turn: {held_chosen / held_best - 1:.2%}.\n")
         f.write("#pragma once\n\nnamespace tab {\n\n")
-        f.write("constexpr int kConvShapes = 7, kConvShapeFeatures = 9;\n")
-        f.write("// rows x filters of the workgroup tile and workgroups a CU holds, per shape\n")
-        f.write("constexpr int kConvShapeTile[kConvShapes][3] = {" + ", ".join("{%d, %d, %d}" % SHAPES[s] for s in range(7)) + "};\n")
+        f.write(f"constexpr int kConvShapes = {len(IDS)}, kConvShapeFeatures = {NFEAT};\n")
+        f.write("// the shape ids tab_set_conv_kernel(TAB_CONV_MATRIX, id) takes, in the order of the tables below\n")
+        f.write("constexpr int kConvShapeIds[kConvShapes] = {" + ", ".join(str(i) for i in IDS) + "};\n")
+        f.write("// rows x filters of the workgroup tile and workgroups a CU holds (compiled occupancy), per shape\n")
+        f.write("constexpr int kConvShapeTile[kConvShapes][3] = {" + ", ".join("{%d, %d, %d}" % SHAPES[s] for s in IDS) + "};\n")
         f.write("constexpr float kConvShapeCost[4][kConvShapes][kConvShapeFeatures] = {\n")
         for t in range(4):
             f.write("    {\n")
-            for s in range(7):
-                f.write("        {" + ", ".join("%.6gf" % v for v in coef[(t, s)]) + "},\n")
+            for s_ in IDS:
+                f.write("        {" + ", ".join(("%.6g" % v if "." in "%.6g" % v or "e" in "%.6g" % v else "%.6g.0" % v) + "f" for v in coef[(t, s_)]) + "},\n")
             f.write("    },\n")
         f.write("};\n\n}  // namespace tab\n")
     print("wrote", out)

@@ -108,6 +108,27 @@ def test_c_abi_rejects_bad_arguments_without_launching():
     assert b"KN" in lib.tab_last_error()
 
 
+def test_conv2d_launches_names_the_one_launch_cases():
+    """tab_conv2d_launches: 1 for a small 1x1 convolution without padding on 64..512 channels (types 0..3), else 2."""
+    lib = _capi.load()
+    p = 4096
+    launches = lambda type, p1, s, N, HW, C, KN, K, x=p: lib.tab_conv2d_launches(x, type, p1, p1, s, s, N, HW, HW, C, KN, K, K)  # noqa: E731
+    assert launches(3, 0, 2, 16, 14, 256, 512, 1) == 1
+    assert launches(0, 0, 1, 4, 28, 64, 100, 1) == 1
+    assert launches(3, 1, 1, 16, 14, 256, 256, 3) == 2      # 3x3
+    assert launches(3, 1, 2, 16, 14, 256, 512, 1) == 2      # padding
+    assert launches(3, 0, 2, 16, 14, 192, 512, 1) == 2      # three words per pixel
+    assert launches(4, 0, 2, 16, 14, 256, 512, 1) == 2      # the CPU-only types
+    assert launches(3, 0, 1, 256, 28, 128, 256, 1) == 2     # a launch too large for it
+    assert launches(3, 0, 2, 16, 14, 256, 512, 1, x=p + 4) == 2  # X not aligned for 16-byte loads
+    assert launches(7, 0, 2, 16, 14, 256, 512, 1) == 0      # bad arguments
+    try:
+        assert lib.tab_set_conv_kernel(1, 2) == 0
+        assert launches(3, 0, 2, 16, 14, 256, 512, 1) == 2  # a forced conv kernel keeps the two launches
+    finally:
+        assert lib.tab_set_conv_kernel(0, -1) == 0
+
+
 def test_set_conv_kernel_validates_without_a_gpu():
     lib = _capi.load()
     try:

@@ -91,3 +91,18 @@ def test_quantize_full_size_properties():
         want, _ = oracle.quantize(xs.reshape(-1, 1, 1, C), t[n_of].numpy(), bitwidth, idx.numel(), 1, 1, C)
         got = q.reshape(N * H * W, C // 64, bitwidth)[idx.cuda()].cpu().numpy()
         assert np.array_equal(got, want.reshape(got.shape))
+
+
+@pytest.mark.parametrize("bitwidth", [1, 2])
+def test_quantize_without_btn(bitwidth):
+    """dev_BTN == NULL (QuantizeActivation): the same packed words, no count vector, for NHWC and NCHW input."""
+    N, H, W, C = 3, 9, 7, 200
+    g = torch.Generator("cpu").manual_seed(bitwidth)
+    x = torch.randn((N, H, W, C), generator=g)
+    ths = (0.7 * x.abs().reshape(N, -1).mean(dim=1)).float() if bitwidth == 2 else torch.zeros(N)
+    want, _ = oracle.quantize(x.numpy(), ths.numpy(), bitwidth, N, H, W, C)
+    got = tab_amd.QuantizeActivation(x.cuda(), ths.cuda(), bitwidth, N, H, W, C)
+    assert np.array_equal(got.cpu().numpy(), want)
+    x_nchw = x.permute(0, 3, 1, 2).contiguous()
+    got = tab_amd.QuantizeActivation(x_nchw.cuda(), ths.cuda(), bitwidth, N, H, W, C, nchw=True)
+    assert np.array_equal(got.cpu().numpy(), want)

@@ -1,0 +1,54 @@
+"""The cost model that picks the matrix-core workgroup shape (tab_conv_shape_model.h, conv_mfma_shape), on the host:
+over a wide grid of geometries, far outside what it was fitted on, every choice is a shape the launch can run and every
+predicted duration is positive, finite and no smaller when K grows."""
+import ctypes
+import itertools
+import math
+
+from tab_amd import _capi
+
+TILE = {0: (128, 128), 1: (128, 64), 2: (64, 64), 3: (32, 32), 4: (256, 64), 5: (256, 128), 6: (128, 256), 8: (64, 64), 9: (128, 128)}
+
+
+def _hook():
+    lib = ctypes.CDLL(_capi.LIB_PATH)
+    f = lib.tab_internal_conv_shape
+    f.restype = ctypes.c_int
+    f.argtypes = [ctypes.c_int] * 6 + [ctypes.POINTER(ctypes.c_float)]
+    return f
+
+
+def _choose(f, type, M, KN, G, PC, packed):
+    cost = ctypes.c_float(-1.0)
+    return f(type, M, KN, G, PC, packed, ctypes.byref(cost)), cost.value
+
+
+def test_every_choice_is_legal_and_priced_positive():
+    f = _hook()
+    Ms = [1, 31, 1024, 12544, 50176, 200704, 1605632, 4096 * 56 * 56, 2**31 - 600]
+    KNs = [1, 63, 64, 100, 512, 1000, 2048, 4096]
+    Ks = [(1, 1), (2, 2), (9, 1), (18, 2), (27, 3), (72, 8), (144, 16), (4096, 64), (65535, 65535)]  # (G, PC)
+    for type, M, KN, (G, PC), packed in itertools.product(range(6), Ms, KNs, Ks, (0, 1)):
+        if packed and type > 3:
+            continue
+        shape, cost = _choose(f, type, M, KN, G, PC, packed)
+        what = (type, M, KN, G, PC, packed, shape, cost)
+        if shape == 7:
+            assert type <= 3 and G <= 9 and packed, what
+            continue
+        assert shape in TILE, what
+        bn = TILE[shape][1]
+        assert bn < 2 * ((KN + 63) // 64 * 64), what          # a filter tile under twice the filters
+        assert not (packed and shape == 3), what              # packed output needs 64-filter tiles
+        assert not (shape >= 8 and PC % 2), what              # split-K shapes: an even number of words per pixel
+        assert math.isfinite(cost) and cost > 0.9, what       # never below a launch
+
+
+def test_predicted_duration_grows_with_k():
+    f = _hook()
+    for type, M, KN in itertools.product((0, 3), (784, 50176, 1605632, 10**8), (64, 512, 4096)):
+        last = 0.0
+        for taps in (1, 4, 9, 25, 49, 400, 4000):
+            _, cost = _choose(f, type, M, KN, taps * 8, 8, 0)
+            assert cost >= last, (type, M, KN, taps, cost, last)
+            last = cost

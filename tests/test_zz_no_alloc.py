@@ -27,13 +27,21 @@ def _both(lib, check, type, N, H, W, C, KN, KH, KW, p1, p2, s1, s2, seed, relu=F
     stream = torch.cuda.current_stream().cuda_stream
     check(lib, lib.tab_conv2d(xd.data_ptr(), QW.data_ptr(), td.data_ptr(), BTN.data_ptr(), type, p1, p2, s1, s2,
                               N, H, W, C, KN, KH, KW, y_ws.data_ptr(), ws.data_ptr(), ws_bytes, stream))
-    # everything the static call touches exists by now: the call itself must not allocate
+    # a first static call looks the scratch's address up (and, like the call above, has the kernels' code loaded):
+    # everything the next one touches exists by then, and that call must not allocate or free, neither through
+    # torch's allocator nor behind its back (the driver's own count of free device memory sees a hipMalloc or
+    # hipFree made inside the library)
+    check(lib, lib.tab_conv2d_static(xd.data_ptr(), QW.data_ptr(), td.data_ptr(), BTN.data_ptr(), type, p1, p2, s1, s2,
+                                     N, H, W, C, KN, KH, KW, y_static.data_ptr(), stream))
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    y_static.fill_(float("nan"))
+    torch.cuda.synchronize()
+    before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
     check(lib, lib.tab_conv2d_static(xd.data_ptr(), QW.data_ptr(), td.data_ptr(), BTN.data_ptr(), type, p1, p2, s1, s2,
                                      N, H, W, C, KN, KH, KW, y_static.data_ptr(), stream))
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before
     assert not torch.isnan(y_static).any()
     assert torch.equal(y_ws, y_static), f"type {type} N={N} {H}x{W}x{C}->{KN} k{KH}x{KW} s{s1}{s2}: outputs differ"
     return y_static
@@ -56,6 +64,36 @@ def test_static_scratch_matches_workspace_on_calls_in_a_row(type):
     qw, btn = oracle.quantize(w.numpy(), w_ths.numpy(), weight_bits(type), 64, 3, 3, 64)
     want = oracle.conv2d(x.numpy(), qw, x_ths.numpy(), btn, type, 1, 0, 1, 1, 1, 8, 8, 64, 64, 3, 3)
     assert np.array_equal(y.cpu().numpy().reshape(want.shape), want)
+
+
+@pytest.mark.parametrize("type", [0, 3])
+def test_static_scratch_under_graph_capture(type):
+    """The use the entry point is made for: captured into a HIP graph after a first eager call, replayed several times
+    with the program's own eager work and synchronisations in between, every replay equal to tab_conv2d's result."""
+    import tab_amd
+    from tab_amd import _capi
+
+    lib = _capi.load()
+    N, H, W, C, KN = 3, 14, 14, 128, 96
+    x, x_ths, w, w_ths = make_layer(type, N, H, W, C, KN, 3, 3, seed=50 + type)
+    QW, BTN = tab_amd.Quantize(w.cuda(), w_ths.cuda(), weight_bits(type), KN, 3, 3, C)
+    xd, td = x.cuda(), x_ths.cuda()
+    want = tab_amd.Conv2d(xd, QW, td, BTN, type, 1, 1, 1, 1, N, H, W, C, KN, 3, 3)
+    out = torch.zeros_like(want)
+    args = (xd.data_ptr(), QW.data_ptr(), td.data_ptr(), BTN.data_ptr(), type, 1, 1, 1, 1, N, H, W, C, KN, 3, 3, out.data_ptr())
+    _capi.check(lib, lib.tab_conv2d_static(*args, torch.cuda.current_stream().cuda_stream))  # address lookup, outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _capi.check(lib, lib.tab_conv2d_static(*args, torch.cuda.current_stream().cuda_stream))
+    for replay in range(4):
+        out.fill_(float("nan"))
+        # eager work that reuses the scratch between the replays: a different, smaller call
+        tab_amd.Conv2dStatic(xd[:1].contiguous(), QW, td[:1].contiguous(), BTN, type, 1, 1, 1, 1, 1, H, W, C, KN, 3, 3)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), f"replay {replay}"
 
 
 def test_static_scratch_formats_4_and_5():
