@@ -172,29 +172,18 @@ __device__ __forceinline__ i32x8 expand_operand(uint32_t p0, uint32_t p1, const 
 // C[8*j + 4*kb + i][r] of the wave's 32x32 tile (mt, nt).  b_nonzero: BTN, bits set in the nonzero plane of
 // the k-positions this lane multiplied, per filter tile; partial: KS * 17 * 64 floats of LDS when the KS
 // waves of the workgroup hold partial sums of one tile.
-template <int TYPE, int TM, int TN, int KCH, int KS, bool BALLOT_PACKING = true>
+template <int TYPE, int TM, int TN, int KCH, int KS>
 __device__ __forceinline__ void conv_mfma_epilogue(const ConvArgs &p, f32x16 (&acc)[TM][TN], int (&b_nonzero)[TN], int wave_m0,
                                                    int wave_n0, int lane, int ks, float *partial)
 {
     const int r = lane & 31, kb = lane >> 5;
-    // btn of this lane's filters (BTN) and, for packed output, the threshold of row r of each 32-row
-    // tile; loaded here rather than before the loop because the registers they would hold through
-    // it push the 128x128 shape over its 128-register budget (requesting them early gained nothing)
+    // btn of this lane's filters (BTN); loaded here rather than before the loop because the registers they would hold
+    // through it push the 128x128 shape over its 128-register budget (requesting them early gained nothing)
     int btn_col[TN];
 #pragma unroll
     for (int nt = 0; nt < TN; nt++) {
         const int col = wave_n0 + nt * 32 + r;
         btn_col[nt] = (TYPE == 2 && col < p.KN) ? p.btn[col] : 0;
-    }
-    float th_row[TM];
-#pragma unroll
-    for (int mt = 0; mt < TM; mt++) {
-        th_row[mt] = 0.f;
-        if (BALLOT_PACKING && p.qy != nullptr) {
-            int n = (int)div32((uint32_t)(wave_m0 + mt * 32 + r), p.div_pixels);
-            n = n < p.N ? n : p.N - 1;  // rows past M are computed but not stored
-            th_row[mt] = p.out_ths[n];
-        }
     }
     if (KS > 1) {
         // the KS waves hold partial sums of the same tile: exchange them through LDS; wave ks
@@ -220,73 +209,6 @@ __device__ __forceinline__ void conv_mfma_epilogue(const ConvArgs &p, f32x16 (&a
         for (int i = 0; i < 4; i++) {
             const int m = wave_m0 + 8 * ks + 4 * kb + i;
             if (col_ok && m < p.M) __builtin_nontemporal_store(sum[i] + bias, &p.y[(size_t)m * p.KN + col]);
-        }
-        return;
-    }
-    if (BALLOT_PACKING && p.qy != nullptr) {
-        // Packed output: Y is not written; each value is thresholded like the quantizer would
-        // threshold it as the next layer's NHWC activation (item = image, channel = filter;
-        // TAB_GEMM.cu:184-192, 231) and a wave ballot is 32 channels of two output pixels: lanes
-        // 0-31 hold row 8j+i, lanes 32-63 row 8j+4+i, so each half of the ballot is one 32-bit
-        // half of a packed word.  Tiles are multiples of 64 filters wide here, so every word that
-        // exists is written completely, tail bits as zeros.
-        const int out_words = (p.KN + 63) >> 6;
-        // lane L (and L+32) holds the threshold of row L of each 32-row tile (th_row) and stores
-        // that row's half-words
-        float bias[TN];
-        bool col_ok[TN];
-#pragma unroll
-        for (int nt = 0; nt < TN; nt++) {
-            const int col = wave_n0 + nt * 32 + r;
-            col_ok[nt] = col < p.KN;
-            bias[nt] = 0.f;
-            if (TYPE == 2) {
-                const int nonzero = b_nonzero[nt] + __shfl_xor(b_nonzero[nt], 32, 64);
-                bias[nt] = (float)(btn_col[nt] - nonzero);
-            }
-            if (TYPE == 3) bias[nt] = (float)(p.num - 64 * p.nchunks * KCH);
-        }
-#pragma unroll
-        for (int mt = 0; mt < TM; mt++) {
-            uint32_t sign_half[TN], nz_half[TN];  // of row r, meaningful in lanes 0-31
-#pragma unroll
-            for (int nt = 0; nt < TN; nt++) sign_half[nt] = nz_half[nt] = 0;
-#pragma unroll
-            for (int j = 0; j < 4; j++)
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int row_lo = 8 * j + i, row_hi = row_lo + 4;  // rows held by lanes 0-31 / 32-63
-                    const float th_lo = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(th_row[mt]), row_lo));
-                    const float th_hi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(th_row[mt]), row_hi));
-                    const float th = kb ? th_hi : th_lo;
-#pragma unroll
-                    for (int nt = 0; nt < TN; nt++) {
-                        const float v = acc[mt][nt][4 * j + i] + bias[nt];
-                        if (p.out_bits == 1) {
-                            const uint64_t b = __ballot(col_ok[nt] && v < th);
-                            sign_half[nt] = r == row_lo ? (uint32_t)b : (r == row_hi ? (uint32_t)(b >> 32) : sign_half[nt]);
-                        } else {
-                            const bool pos = v > th, neg = !pos && v < -th;
-                            const uint64_t sg = __ballot(col_ok[nt] && neg), nz = __ballot(col_ok[nt] && (pos || neg));
-                            sign_half[nt] = r == row_lo ? (uint32_t)sg : (r == row_hi ? (uint32_t)(sg >> 32) : sign_half[nt]);
-                            nz_half[nt] = r == row_lo ? (uint32_t)nz : (r == row_hi ? (uint32_t)(nz >> 32) : nz_half[nt]);
-                        }
-                    }
-                }
-            const int m = wave_m0 + mt * 32 + r;
-#pragma unroll
-            for (int nt = 0; nt < TN; nt++) {
-                const int col0 = wave_n0 + nt * 32;  // uniform
-                if (col0 >= 64 * out_words || lane >= 32 || m >= p.M) continue;
-                const size_t word = (size_t)m * out_words + (col0 >> 6);
-                const int half = (col0 >> 5) & 1;
-                if (p.out_bits == 1) {
-                    p.qy[word * 2 + half] = sign_half[nt];
-                } else {
-                    p.qy[(word * 2 + 0) * 2 + half] = sign_half[nt];
-                    p.qy[(word * 2 + 1) * 2 + half] = nz_half[nt];
-                }
-            }
         }
         return;
     }
@@ -334,8 +256,8 @@ __device__ __forceinline__ void conv_mfma_epilogue(const ConvArgs &p, f32x16 (&a
 // pixel.  It thresholds them against that pixel's threshold (a per-lane constant) exactly as the quantizer would
 // threshold them as the next layer's NHWC activation (item = image, channel = filter; TAB_GEMM.cu:184-192, 231) into 16
 // bits, and the other half-wave's lane of the same pixel supplies the other 16 of the 32-bit half word: no ballot and
-// no cross-lane deposit per value (the ballot form above costs about 13 vector instructions per pair of rows, this
-// one 2-3 per value).  The per-filter bias of BTN (btn - nonzero weights, known per lane = filter after the loop) is
+// no cross-lane deposit per value (packing by wave ballot, with the activation as the first operand, costs about 13 vector
+// instructions per pair of rows, this 2-3 per value).  The per-filter bias of BTN (btn - nonzero weights, known per lane = filter after the loop) is
 // handed to the lanes that need it through `exchange`, 32*TN dwords of LDS private to the wave.
 template <int TYPE, int TM, int TN, int KCH>
 __device__ __forceinline__ void conv_mfma_epilogue_packed(const ConvArgs &p, f32x16 (&acc)[TM][TN], int (&b_nonzero)[TN], int wave_m0,
@@ -503,11 +425,13 @@ constexpr int conv_mfma_lds_bytes()
     return 4 * (2 * (Stager::A_DWORDS + Stager::B_DWORDS) + (KS > 1 ? KS * 17 * 64 : 1));
 }
 
-template <int TYPE, int WM, int WN, int TM, int TN, int KCH, bool INTAP, int KS = 1>
+// PACKED: packed output (p.qy): the weights are the first MFMA operand and the epilogue packs inside a lane.
+template <int TYPE, int WM, int WN, int TM, int TN, int KCH, bool INTAP, int KS = 1, bool PACKED = false>
 __global__ __launch_bounds__(kConvThreads)
 __attribute__((amdgpu_waves_per_eu(mfma_waves_per_eu(WM, TM, TN, conv_mfma_lds_bytes<TYPE, WM, WN, TM, TN, KCH, INTAP, KS>())))) void conv_mfma(const ConvArgs p)
 {
     static_assert(WM * WN * KS * 64 == kConvThreads, "four waves");
+    static_assert(!PACKED || (KS == 1 && TYPE <= 3), "packed output: whole tiles per wave, types 0..3");
     static_assert(KCH % KS == 0 && (KS == 1 || (TM == 1 && TN == 1)), "k-split waves share one 32x32 tile");
     constexpr int WPW = KCH / KS;  // words of a chunk each wave multiplies
     constexpr int APL = Planes<TYPE>::A, BPL = Planes<TYPE>::B;
@@ -604,7 +528,8 @@ __attribute__((amdgpu_waves_per_eu(mfma_waves_per_eu(WM, TM, TN, conv_mfma_lds_b
             for (int mt = 0; mt < TM; mt++)
 #pragma unroll
                 for (int nt = 0; nt < TN; nt++)
-                    acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[mt], bf[nt], acc[mt][nt], 4, 4, 0, 0, 0, 0);
+                    acc[mt][nt] = PACKED ? __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[nt], af[mt], acc[mt][nt], 4, 4, 0, 0, 0, 0)
+                                         : __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[mt], bf[nt], acc[mt][nt], 4, 4, 0, 0, 0, 0);
         }
 
         if (more) st.stage(lds + ((chunk + 1) & 1) * (A_DWORDS + B_DWORDS));
@@ -612,7 +537,10 @@ __attribute__((amdgpu_waves_per_eu(mfma_waves_per_eu(WM, TM, TN, conv_mfma_lds_b
     }
 
     scale_ternary_sums<TYPE>(acc);
-    conv_mfma_epilogue<TYPE, TM, TN, KCH, KS>(p, acc, b_nonzero, wave_m0, wave_n0, lane, ks, partial);
+    if constexpr (PACKED)  // (the chunk loop ends on a barrier: the operand buffers are free for BTN's exchange of biases)
+        conv_mfma_epilogue_packed<TYPE, TM, TN, KCH>(p, acc, b_nonzero, wave_m0, wave_n0, lane, lds + wave * (32 * TN));
+    else
+        conv_mfma_epilogue<TYPE, TM, TN, KCH, KS>(p, acc, b_nonzero, wave_m0, wave_n0, lane, ks, partial);
 }
 
 // Chunk length for G words: 1..4, the one with the least padded work (a barrier is priced as half a
@@ -636,7 +564,14 @@ hipError_t launch_mfma_tile(ConvArgs a, hipStream_t stream)
     a.tiles_m = (a.M + BM - 1) / BM;
     const long blocks = order_workgroups<Planes<TYPE>::A>(a, (a.KN + BN - 1) / BN);
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
-    conv_mfma<TYPE, WM, WN, TM, TN, KCH, INTAP, KS><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
+    if (a.qy != nullptr) {
+        if constexpr (TYPE <= 3 && KS == 1)
+            conv_mfma<TYPE, WM, WN, TM, TN, KCH, INTAP, KS, true><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
+        else
+            return hipErrorInvalidValue;  // no packed output for types 4 and 5, nor from the k-split 32x32 shape
+    } else {
+        conv_mfma<TYPE, WM, WN, TM, TN, KCH, INTAP, KS><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
+    }
     return hipGetLastError();
 }
 

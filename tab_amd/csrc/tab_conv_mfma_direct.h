@@ -401,7 +401,7 @@ __attribute__((amdgpu_waves_per_eu(mfma_waves_per_eu(KS > 1 ? 1 : WM, TM, TN, 4 
                 if constexpr (PACKED)
                     conv_mfma_epilogue_packed<TYPE, 1, 1, KCH>(p, sum, nonzero, wave_m0 + mt * 32, wave_n0 + nt * 32, lane, exchange);
                 else
-                    conv_mfma_epilogue<TYPE, 1, 1, KCH, 1, false>(p, sum, nonzero, wave_m0 + mt * 32, wave_n0 + nt * 32, lane, 0, nullptr);
+                    conv_mfma_epilogue<TYPE, 1, 1, KCH, 1>(p, sum, nonzero, wave_m0 + mt * 32, wave_n0 + nt * 32, lane, 0, nullptr);
             }
             if (round + 1 < NT / RT) __syncthreads();  // the parts are read before the next round overwrites them
         }
@@ -411,7 +411,7 @@ __attribute__((amdgpu_waves_per_eu(mfma_waves_per_eu(KS > 1 ? 1 : WM, TM, TN, 4 
         if (TYPE == 2) __syncthreads();
         conv_mfma_epilogue_packed<TYPE, TM, TN, KCH>(p, acc, b_nonzero, wave_m0, wave_n0, lane, lds + wave * (32 * TN));
     } else {
-        conv_mfma_epilogue<TYPE, TM, TN, KCH, 1, false>(p, acc, b_nonzero, wave_m0, wave_n0, lane, 0, nullptr);
+        conv_mfma_epilogue<TYPE, TM, TN, KCH, 1>(p, acc, b_nonzero, wave_m0, wave_n0, lane, 0, nullptr);
     }
 }
 
