@@ -105,11 +105,15 @@ int tab_internal_conv_shape(int type, int M, int KN, int G, int PC, int packed, 
     return tab::conv_mfma_shape(type, a, cost_us);
 }
 
+/* Test hook, absent from include/tab_amd.h: the number of workgroups the mixed launch (TAB_CONV_MATRIX tile 10) counts as one
+ * round of the chip; 0 = the device's compute units.  Small values let small test shapes mix whole tiles and quarters. */
+void tab_internal_set_tail_round(int workgroups) { tab::set_tail_round(workgroups); }
+
 int tab_set_conv_kernel(int kernel, int tile)
 {
     static const int popcount_tm[4] = {7, 8, 4, 2};  // 7: the popcount kernel's own choice
     if (kernel == TAB_CONV_AUTO && tile == -1) tab::force_conv_tile(0, 0);
-    else if (kernel == TAB_CONV_MATRIX && tile >= -1 && tile <= 9) tab::force_conv_tile(9, tile);
+    else if (kernel == TAB_CONV_MATRIX && tile >= -1 && tile <= 10) tab::force_conv_tile(9, tile);
     else if (kernel == TAB_CONV_POPCOUNT && tile >= -1 && tile <= 2) tab::force_conv_tile(popcount_tm[tile + 1], 0);
     else return fail(TAB_ERR_BAD_ARGUMENT, "no conv kernel %d with tile %d", kernel, tile);
     return TAB_OK;
@@ -253,7 +257,7 @@ static int conv_packed(const int64_t *dev_QX, const int64_t *dev_QW, const int32
     a.div_ow = tab::make_div32((uint32_t)s.OW);
     a.div_tiles_m = tab::make_div32(1);
     a.tiles_n = 0;
-    a.xcd_share = 0; a.filter_tiles = 1;
+    a.xcd_share = 0; a.filter_tiles = 1; a.tail_big = 0;
     // A Y that fits the 256 MB last-level cache beside the operands but not the L2s is written through the caches
     // (the cache takes the stores faster than HBM: Y of 190-206 MB 1-11 % sooner); every other Y with non-temporal
     // stores: a smaller one leaves no dirty L2 to flush when the launch ends (7-25 % sooner), a larger one would only

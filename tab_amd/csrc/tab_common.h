@@ -74,6 +74,7 @@ struct ConvArgs {
     int xcd_share;      // tiles each of the 8 XCDs takes as one contiguous run of rows of Y (0: order not XCD-aware)
     int filter_tiles;   // ceil(KN / BN), with div_filter_tiles, for that order
     Div32 div_filter_tiles;
+    int tail_big;       // the mixed launch (conv_mfma_tail): workgroups that take whole 128x128 tiles; the rest take quarters
     FastDiv div_pc, div_kw;
     Div32 div_pixels, div_ow;  // by OH*OW and OW: an output row's image and line
 };
@@ -125,6 +126,8 @@ hipError_t launch_conv1x1_fused(int type, const float *x, const float *ths, cons
                                 int H, int W, int C, int KN, int s1, int s2, int OH, int OW, hipStream_t stream);
 
 void force_conv_tile(int tm, int ng);  // tuning hook: 0,0 restores the automatic choice
+void set_tail_round(int workgroups);   // test hook of the mixed launch: workgroups counted as one round of the chip (0: the CUs)
+int tail_round();
 bool conv_kernel_forced();             // true while tab_set_conv_kernel holds a choice other than the automatic one
 
 }  // namespace tab

@@ -360,6 +360,14 @@ int device_compute_units()
     return cus;
 }
 
+std::atomic<int> g_tail_round{0};
+void set_tail_round(int workgroups) { g_tail_round.store(workgroups > 0 ? workgroups : 0, std::memory_order_relaxed); }
+int tail_round()
+{
+    const int forced = g_tail_round.load(std::memory_order_relaxed);
+    return forced > 0 ? forced : device_compute_units();
+}
+
 bool conv_kernel_forced() { return g_forced_kernel.load(std::memory_order_relaxed) != 0; }
 
 // fp32 accumulators hold integers up to 2^24 exactly; a product is at most 1 (9 for the 2-bit levels of
@@ -417,14 +425,25 @@ int conv_mfma_shape(int conv_type, const ConvArgs &a, float *cost_us)
         if (shape == 3 && a.qy != nullptr) continue;        // the packed epilogues need tiles 64 filters wide
         if (shape >= 8 && a.PC % 2 != 0) continue;          // the split-K shapes move whole pairs of words inside a tap
         const long tiles = (long)((a.M + bm - 1) / bm) * ((a.KN + bn - 1) / bn);
-        const float n = (float)((tiles + cus - 1) / cus), rounds = (float)(((tiles + cus - 1) / cus + held - 1) / held);
-        const float busy = tiles >= cus ? 1.f : (float)tiles / (float)cus;
-        const float f[kConvShapeFeatures] = {(float)a.G * n, (float)a.G * rounds, rounds, n, y_mb, y_mb * busy, busy, 1.f,
-                                             a.G <= 9 ? y_mb : 0.f};
-        float cost = 0.f;
-        for (int k = 0; k < kConvShapeFeatures; k++) cost += kConvShapeCost[type][i][k] * f[k];
-        // the busiest CU's n tiles of (bm/32)(bn/32) MFMA tiles x G words, 32 cycles each on four SIMDs at 2.4 GHz, and a launch
-        const float floor_us = 1.f + n * (float)(bm / 32 * (bn / 32)) * (float)a.G * (32.f / 4.f / 2400.f);
+        float cost = 0.f, floor_us;
+        if (shape == 10) {
+            // the mixed launch: whole tiles on every CU, then quarter tiles; a candidate where it has both, the words per
+            // pixel come in fours and K is more than nine words (with a shorter K the launch is its epilogue)
+            const long whole = tiles / cus, quarters = (4 * (tiles % cus) + cus - 1) / cus;
+            if (a.PC % 4 != 0 || a.G <= 9 || whole == 0 || quarters == 0) continue;
+            const float f[kConvShapeFeatures] = {(float)a.G * (float)whole, (float)a.G * (float)quarters, (float)quarters, (float)whole, y_mb, y_mb,
+                                                 1.f, 1.f, 0.f};
+            for (int k = 0; k < kConvShapeFeatures; k++) cost += kConvShapeCost[type][i][k] * f[k];
+            floor_us = 1.f + (float)(16 * whole + 4 * quarters) * (float)a.G * (32.f / 4.f / 2400.f);
+        } else {
+            const float n = (float)((tiles + cus - 1) / cus), rounds = (float)(((tiles + cus - 1) / cus + held - 1) / held);
+            const float busy = tiles >= cus ? 1.f : (float)tiles / (float)cus;
+            const float f[kConvShapeFeatures] = {(float)a.G * n, (float)a.G * rounds, rounds, n, y_mb, y_mb * busy, busy, 1.f,
+                                                 a.G <= 9 ? y_mb : 0.f};
+            for (int k = 0; k < kConvShapeFeatures; k++) cost += kConvShapeCost[type][i][k] * f[k];
+            // the busiest CU's n tiles of (bm/32)(bn/32) MFMA tiles x G words, 32 cycles each on four SIMDs at 2.4 GHz, and a launch
+            floor_us = 1.f + n * (float)(bm / 32 * (bn / 32)) * (float)a.G * (32.f / 4.f / 2400.f);
+        }
         if (cost < floor_us) cost = floor_us;
         if (!any || cost < best_cost) {
             any = true;
@@ -442,7 +461,7 @@ hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream)
     const int force_tm = forced.tm, force_ng = forced.ng;
     if (args.qy != nullptr) {  // packed output exists in the matrix-core kernel's 64-wide shapes only
         if (!conv_mfma_exact(args)) return hipErrorInvalidValue;
-        const int shape = (force_tm == 9 && force_ng >= 0 && force_ng != 3 && force_ng <= 9) ? force_ng : conv_mfma_shape(type, args);
+        const int shape = (force_tm == 9 && force_ng >= 0 && force_ng != 3 && force_ng <= 10) ? force_ng : conv_mfma_shape(type, args);
         return launch_conv_mfma(type, args, shape, stream);
     }
     if (force_tm == 9) return launch_conv_mfma(type, args, force_ng < 0 ? conv_mfma_shape(type, args) : force_ng, stream);

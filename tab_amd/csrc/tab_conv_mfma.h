@@ -168,6 +168,11 @@ __device__ __forceinline__ i32x8 expand_operand(uint32_t p0, uint32_t p1, const 
     return r;
 }
 
+// Words of K a kernel with chunks of KCH words multiplies: K rounded up to whole chunks (the words past K are zeros, which add
+// +64 each for binary x binary: the BNN bias counts them).
+template <int KCH>
+__device__ __forceinline__ int padded_words(const ConvArgs &p) { return (p.G + KCH - 1) / KCH * KCH; }
+
 // Epilogue shared by the matrix-core kernels: accumulator element 4*j + i of lane (kb, r) is
 // C[8*j + 4*kb + i][r] of the wave's 32x32 tile (mt, nt).  b_nonzero: BTN, bits set in the nonzero plane of
 // the k-positions this lane multiplied, per filter tile; partial: KS * 17 * 64 floats of LDS when the KS
@@ -204,7 +209,7 @@ __device__ __forceinline__ void conv_mfma_epilogue(const ConvArgs &p, f32x16 (&a
         const bool col_ok = col < p.KN;
         float bias = 0.f;
         if (TYPE == 2) bias = (float)btn_col[0] - (sum[4] + __shfl_xor(sum[4], 32, 64));
-        if (TYPE == 3) bias = (float)(p.num - 64 * p.nchunks * KCH);
+        if (TYPE == 3) bias = (float)(p.num - 64 * padded_words<KCH>(p));
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const int m = wave_m0 + 8 * ks + 4 * kb + i;
@@ -231,7 +236,7 @@ __device__ __forceinline__ void conv_mfma_epilogue(const ConvArgs &p, f32x16 (&a
             const int nonzero = b_nonzero[nt] + __shfl_xor(b_nonzero[nt], 32, 64);
             bias = (float)(btn_col[nt] - nonzero);
         }
-        if (TYPE == 3) bias = (float)(p.num - 64 * p.nchunks * KCH);
+        if (TYPE == 3) bias = (float)(p.num - 64 * padded_words<KCH>(p));
         // kNoFilter + any offset inside the tile stays out of range without wrapping
         const uint32_t lane_off = col < p.KN ? (uint32_t)(4 * kb) * row_bytes + (uint32_t)col * 4u : kNoFilter;
         auto store_tiles = [&](auto policy) {
@@ -292,7 +297,7 @@ __device__ __forceinline__ void conv_mfma_epilogue_packed(const ConvArgs &p, f32
             if (TYPE == 2) v = *reinterpret_cast<const u32x4 *>(exchange + nt * 32 + 8 * j + 4 * kb);
 #pragma unroll
             for (int i = 0; i < 4; i++)
-                bias[nt][4 * j + i] = TYPE == 2 ? __uint_as_float(v[i]) : (TYPE == 3 ? (float)(p.num - 64 * p.nchunks * KCH) : 0.f);
+                bias[nt][4 * j + i] = TYPE == 2 ? __uint_as_float(v[i]) : (TYPE == 3 ? (float)(p.num - 64 * padded_words<KCH>(p)) : 0.f);
         }
 
     auto pack_rows = [&](auto out_bits_constant) {
@@ -582,6 +587,8 @@ template <int TYPE, int WM, int WN, int TM, int TN, int KCH, int KS = 1, int ARU
 hipError_t launch_mfma_direct(ConvArgs a, hipStream_t stream);
 template <int TYPE, int WM, int WN, int TM, int TN, int KS, int WORDS>
 hipError_t launch_mfma_split(const ConvArgs &a, hipStream_t stream);
+template <int TYPE>
+hipError_t launch_mfma_tail(ConvArgs a, hipStream_t stream);
 
 template <int TYPE, int WM, int WN, int TM, int TN, int KCH, int KS = 1>
 hipError_t launch_mfma_intap(const ConvArgs &a, hipStream_t stream)
@@ -633,7 +640,8 @@ hipError_t launch_mfma_regs(const ConvArgs &a, hipStream_t stream);
 // short-K kernel (K of at most nine words; longer K falls back to the shape picked from the launch),
 // 8 = 64x64 with K split over the four waves (each wave 2x2 MFMA tiles over a quarter of every chunk), 9 = 128x128 with K
 // split over two pairs of waves (each wave 2x4 MFMA tiles over half of every chunk); both need an even number of words per
-// pixel and otherwise run as shapes 2 and 0
+// pixel and otherwise run as shapes 2 and 0, 10 = 128x128 tiles for the whole rounds of the chip and 64x64 split-K quarters for
+// the rest of the last round (words per pixel in fours; otherwise shape 0)
 template <int TYPE>
 hipError_t launch_mfma_type(const ConvArgs &a, int shape, hipStream_t stream)
 {
@@ -642,6 +650,10 @@ hipError_t launch_mfma_type(const ConvArgs &a, int shape, hipStream_t stream)
             if (a.G <= 9) return launch_mfma_regs<TYPE>(a, stream);
         shape = conv_mfma_shape(TYPE, a);
         if (shape == 7) return hipErrorInvalidValue;
+    }
+    if (shape == 10) {
+        if (a.PC % 4 == 0) return launch_mfma_tail<TYPE>(a, stream);
+        shape = 0;
     }
     if (shape == 8 && a.PC % 2 != 0) shape = 2;
     if (shape == 9 && a.PC % 2 != 0) shape = 0;

@@ -74,9 +74,10 @@ constexpr int conv_mfma_direct_lds_dwords()
     return buffers > split ? buffers : split;
 }
 
-template <int TYPE, int WM, int WN, int TM, int TN, int KCH, bool PACKED, int KS = 1, int ARUN = 0>
-__global__ __launch_bounds__(kConvThreads)
-__attribute__((amdgpu_waves_per_eu(mfma_waves_per_eu(KS > 1 ? 1 : WM, TM, TN, 4 * conv_mfma_direct_lds_dwords<TYPE, WM, WN, TM, TN, KCH, KS>())))) void conv_mfma_direct(const ConvArgs p)
+// One tile of Y, by the whole workgroup: tile (tile_m, tile_n) of the launch's BM x BN grid, operands through the
+// workgroup's LDS `lds` (conv_mfma_direct_lds_dwords<...>() dwords).
+template <int TYPE, int WM, int WN, int TM, int TN, int KCH, bool PACKED, int KS, int ARUN>
+__device__ __forceinline__ void conv_mfma_direct_tile(const ConvArgs &p, uint32_t *lds, int tile_m, int tile_n)
 {
     static_assert(WM * WN * KS * 64 == kConvThreads && KCH % (2 * KS) == 0, "four waves, whole pairs of words per wave group");
     constexpr int PAIRS = KCH / 2;
@@ -90,7 +91,7 @@ __attribute__((amdgpu_waves_per_eu(mfma_waves_per_eu(KS > 1 ? 1 : WM, TM, TN, 4 
     constexpr int A_RUN = ARUN ? ARUN : granule_run(PA, APL), B_RUN = granule_run(PB, BPL);
     static_assert(BM % 64 == 0 && BN % 64 == 0, "one wave instruction moves 64 / RUN rows of one run");
     static_assert(PA % A_RUN == 0, "whole runs");
-    __shared__ __attribute__((aligned(16))) uint32_t lds[conv_mfma_direct_lds_dwords<TYPE, WM, WN, TM, TN, KCH, KS>()];
+    const int nchunks = (p.G + KCH - 1) / KCH;  // (the split-K shapes fetch the words past K as zeros)
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -101,8 +102,6 @@ __attribute__((amdgpu_waves_per_eu(mfma_waves_per_eu(KS > 1 ? 1 : WM, TM, TN, 4 
     const size_t image_words = (size_t)p.H * p.W * p.PC * APL;
     const size_t filter_bytes = (size_t)p.G * BPL * 8;
 
-    int tile_m, tile_n;
-    if (!tile_of_workgroup(p, tile_m, tile_n)) return;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
     // ---- what this lane fetches: granule idx = tid + i * 256 = (run * ROWS + row) * RUN + column ------
@@ -279,8 +278,8 @@ __attribute__((amdgpu_waves_per_eu(mfma_waves_per_eu(KS > 1 ? 1 : WM, TM, TN, 4 
         for (int q = 0; q < 4 * NE; q++) expand_piece(q, 0, 0, 0);
     }
 
-    for (int chunk = 0; chunk < p.nchunks; chunk++) {
-        const bool more = chunk + 1 < p.nchunks;
+    for (int chunk = 0; chunk < nchunks; chunk++) {
+        const bool more = chunk + 1 < nchunks;
         const uint32_t *buf = lds + (chunk & 1) * BUF_DWORDS;
         uint32_t *next = lds + ((chunk + 1) & 1) * BUF_DWORDS;
 
@@ -413,6 +412,81 @@ __attribute__((amdgpu_waves_per_eu(mfma_waves_per_eu(KS > 1 ? 1 : WM, TM, TN, 4 
     } else {
         conv_mfma_epilogue<TYPE, TM, TN, KCH, 1>(p, acc, b_nonzero, wave_m0, wave_n0, lane, 0, nullptr);
     }
+}
+
+template <int TYPE, int WM, int WN, int TM, int TN, int KCH, bool PACKED, int KS = 1, int ARUN = 0>
+__global__ __launch_bounds__(kConvThreads)
+__attribute__((amdgpu_waves_per_eu(mfma_waves_per_eu(KS > 1 ? 1 : WM, TM, TN, 4 * conv_mfma_direct_lds_dwords<TYPE, WM, WN, TM, TN, KCH, KS>())))) void conv_mfma_direct(const ConvArgs p)
+{
+    __shared__ __attribute__((aligned(16))) uint32_t lds[conv_mfma_direct_lds_dwords<TYPE, WM, WN, TM, TN, KCH, KS>()];
+    int tile_m, tile_n;
+    if (!tile_of_workgroup(p, tile_m, tile_n)) return;
+    conv_mfma_direct_tile<TYPE, WM, WN, TM, TN, KCH, PACKED, KS, ARUN>(p, lds, tile_m, tile_n);
+}
+
+// Mixed launch for grids of a few rounds of the chip: a launch lasts as long as its busiest CU, and with T tiles on C CUs that
+// is ceil(T / C) tiles although the mean is T / C (392 tiles of 128x128 on 256 CUs: two against 1.53; 784: four against 3.06).
+// Here the first floor(T / C) * C workgroups take whole 128x128 tiles (four MFMA tiles a wave, chunks of four words) and the
+// remaining tiles are cut into four 64x64 quarters each, run by the split-K body (the large tile's ratio of expansions to
+// MFMAs): the last, partial round is dealt out in quarters, so the busiest CU carries at most a quarter tile more than the
+// others.  Workgroups are dispatched in index order, whole tiles first.  Needs words per pixel in fours (PC % 4 == 0).
+template <int TYPE, int ARUN, bool PACKED>
+__global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(4))) void conv_mfma_tail(const ConvArgs p)
+{
+    constexpr int BIG = conv_mfma_direct_lds_dwords<TYPE, 2, 2, 2, 2, 4, 1>(), SMALL = conv_mfma_direct_lds_dwords<TYPE, 1, 1, 2, 2, 8, 4>();
+    __shared__ __attribute__((aligned(16))) uint32_t lds[BIG > SMALL ? BIG : SMALL];
+    const uint32_t b = blockIdx.x;
+    if (b < (uint32_t)p.tail_big) {  // uniform over the workgroup
+        // XCD-aware order over the whole tiles, as in tile_of_workgroup
+        const uint32_t logical = b < 8u * (uint32_t)p.xcd_share ? (b & 7u) * (uint32_t)p.xcd_share + (b >> 3) : b;
+        const int tile_m = (int)div32(logical, p.div_filter_tiles);
+        conv_mfma_direct_tile<TYPE, 2, 2, 2, 2, 4, PACKED, 1, 0>(p, lds, tile_m, (int)logical - tile_m * p.filter_tiles);
+    } else {
+        const uint32_t j = b - (uint32_t)p.tail_big, t = (uint32_t)p.tail_big + (j >> 2), q = j & 3u;
+        const int big_m = (int)div32(t, p.div_filter_tiles), big_n = (int)t - big_m * p.filter_tiles;
+        const int tile_m = 2 * big_m + (int)(q & 1u), tile_n = 2 * big_n + (int)(q >> 1);
+        if (tile_m * 64 >= p.M || tile_n * 64 >= p.KN) return;  // a quarter wholly past the edge of Y
+        conv_mfma_direct_tile<TYPE, 1, 1, 2, 2, 8, PACKED, 4, ARUN>(p, lds, tile_m, tile_n);
+    }
+}
+
+template <int TYPE, int ARUN>
+hipError_t launch_mfma_tail_run(ConvArgs a, long blocks, hipStream_t stream)
+{
+    if (a.qy != nullptr) {
+        if constexpr (TYPE <= 3)
+            conv_mfma_tail<TYPE, ARUN, true><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
+        else
+            return hipErrorInvalidValue;  // no packed output for types 4 and 5
+    } else {
+        conv_mfma_tail<TYPE, ARUN, false><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
+    }
+    return hipGetLastError();
+}
+
+// False when the layer does not fit the mixed launch (words per pixel not in fours).
+inline bool mfma_tail_supported(const ConvArgs &a) { return a.PC % 4 == 0; }
+
+template <int TYPE>
+hipError_t launch_mfma_tail(ConvArgs a, hipStream_t stream)
+{
+    if (!mfma_tail_supported(a)) return hipErrorInvalidValue;
+    const long filter_tiles = (a.KN + 127) / 128, tiles = (long)((a.M + 127) / 128) * filter_tiles;
+    const long round = tail_round();
+    const long whole = tiles / round * round;
+    const long blocks = whole + 4 * (tiles - whole);
+    if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
+    a.kcw = 4;
+    a.nchunks = a.G / 4;
+    a.tiles_m = (a.M + 127) / 128;
+    a.tiles_n = 0;
+    a.tail_big = (int)whole;
+    a.filter_tiles = (int)filter_tiles;
+    a.div_filter_tiles = make_div32((uint32_t)filter_tiles);
+    a.xcd_share = whole >= 64 ? (int)(whole / 8) : 0;
+    // granules of an activation pixel: runs of four where the pixel has them, else of two (one-plane operands on 256 channels)
+    if (a.PC * Planes<TYPE>::A / 2 % 4 == 0) return launch_mfma_tail_run<TYPE, 4>(a, blocks, stream);
+    return launch_mfma_tail_run<TYPE, 2>(a, blocks, stream);
 }
 
 template <int TYPE, int WM, int WN, int TM, int TN, int KCH, int KS, int ARUN>

@@ -11,6 +11,12 @@ Model, per (type, shape): duration ~ c . f with the features
     busy   = min(1, tiles / 256)                     share of the CUs that have work at all
     G      = KH*KW*PC words of K, Y = 4*M*KN bytes / 1e6; the last feature gives the layers whose loop is a handful of
              MFMAs (C = 64 with 3x3, 1x1) their own price per byte of Y: their launches are the epilogue
+The mixed launch (shape 10: 128x128 tiles for the whole rounds of the chip, 64x64 split-K quarters for the rest) has
+    f = [G*whole, G*quarters, quarters, whole, Y, Y, 1, 1, Y*[G <= 9]]
+    whole    = floor(tiles / 256)                    whole tiles on every CU
+    quarters = ceil(4 * (tiles mod 256) / 256)       quarter tiles on the busiest CU after them
+and is a candidate where both are positive, the words per pixel come in fours and K is more than nine words (with a
+shorter K the launch is its epilogue, and the large tile alone writes Y in the better order).
 fitted by NON-NEGATIVE least squares on relative error (the N=16 set weighted threefold): every feature is non-negative and
 so is every coefficient, hence a predicted duration is positive and grows with K, with the tiles on the busiest CU and
 with Y for every geometry, inside the fitted range or far outside it (an unconstrained fit had coefficients of both signs,
@@ -29,7 +35,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 # shape id -> rows x filters of the workgroup tile, workgroups a CU holds (the occupancy the compiler reports for the
 # shape's kernels with four-word chunks: registers, or LDS where that is the tighter limit)
 SHAPES = {0: (128, 128, 4), 1: (128, 64, 6), 2: (64, 64, 8), 3: (32, 32, 4), 4: (256, 64, 4), 5: (256, 128, 2), 6: (128, 256, 2),
-          8: (64, 64, 4), 9: (128, 128, 2)}
+          8: (64, 64, 4), 9: (128, 128, 2), 10: (128, 128, 4)}
+MIXED = 10
 IDS = sorted(SHAPES)
 NFEAT = 9
 
@@ -51,18 +58,28 @@ def parse(path):
     return rows
 
 
+def mixed_rounds(r):
+    tiles = -(-r["M"] // 128) * -(-r["KN"] // 128)
+    return tiles // 256, -(-4 * (tiles % 256) // 256)
+
+
 def eligible(r, s):
     # (the split-K shapes need an even number of words per pixel; otherwise they run as shapes 2 and 0)
+    if s == MIXED and (r["PC"] % 4 or r["G"] <= 9 or 0 in mixed_rounds(r)):
+        return False
     return SHAPES[s][1] < 2 * (-(-r["KN"] // 64) * 64) and s in r["times"] and not (s >= 8 and r["PC"] % 2)
 
 
 def features(r, s):
     BM, BN, held = SHAPES[s]
+    Y = r["M"] * r["KN"] * 4e-6
+    if s == MIXED:
+        whole, quarters = mixed_rounds(r)
+        return [r["G"] * whole, r["G"] * quarters, quarters, whole, Y, Y, 1.0, 1.0, Y if r["G"] <= 9 else 0.0]
     tiles = -(-r["M"] // BM) * -(-r["KN"] // BN)
     n = -(-tiles // 256)
     rounds = -(-n // held)
     busy = min(1.0, tiles / 256.0)
-    Y = r["M"] * r["KN"] * 4e-6
     return [r["G"] * n, r["G"] * rounds, rounds, n, Y, Y * busy, busy, 1.0, Y if r["G"] <= 9 else 0.0]
 
 
@@ -84,11 +101,15 @@ def choose(coef, r):
     return min((s for s in SHAPES if eligible(r, s)), key=lambda s: (float(coef[(r["type"], s)] @ np.array(features(r, s))), s))
 
 
+def best_time(r):
+    return min(v for s, v in r["times"].items() if eligible(r, s))
+
+
 def regret(rows, coef):
     chosen = best = 0.0
     per = collections.defaultdict(lambda: [0.0, 0.0])
     for r in rows:
-        c, b = r["times"][choose(coef, r)], min(r["times"].values())
+        c, b = r["times"][choose(coef, r)], best_time(r)
         chosen += c
         best += b
         per[r["set"]][0] += c
@@ -110,7 +131,7 @@ def main():
         for r in rows:
             if r["set"] == hold:
                 held_chosen += r["times"][choose(c, r)]
-                held_best += min(r["times"].values())
+                held_best += best_time(r)
     print(f"{len(rows)} cases; regret of the model's choice, fitted on all: {total:.2%} ({', '.join(f'{k} {v:.1%}' for k, v in sorted(per.items()))})")
     print(f"each set held out of the fit in turn: {held_chosen / held_best - 1:.2%} ({', '.join(f'{k} {v:.1%}' for k, v in sorted(held.items()))})")
     out = os.path.join(os.path.dirname(HERE), "csrc", "tab_conv_shape_model.h")
@@ -123,7 +144,8 @@ def main():
         f.write(f"// Fitted {datetime.date.today().isoformat()} on the kernels of commit {commit} (and the working tree on top of it).\n")
         f.write("// Cost model of the matrix-core workgroup shapes: predicted duration (us) = kConvShapeCost[type][i] . f for the shape\n")
         f.write("// kConvShapeIds[i], f = {G*n, G*rounds, rounds, n, Y, Y*busy, busy, 1, Y*[G <= 9]} (n = tiles on the busiest CU,\n")
-        f.write("// rounds = refills of that CU, Y = megabytes of output, busy = share of the CUs with work).  Non-negative least squares:\n")
+        f.write("// rounds = refills of that CU, Y = megabytes of output, busy = share of the CUs with work; shape 10, the mixed launch:\n")
+        f.write("// {G*whole, G*quarters, quarters, whole, Y, Y, 1, 1, Y*[G <= 9]}, whole tiles per CU and quarter tiles after them).  Non-negative least squares:\n")
         f.write("// every feature and every coefficient is >= 0, so a prediction is positive and monotone for any geometry.  Regret of the\n")
         f.write(f"// choice against the best measured shape over the {len(rows)} fitted cases: {total:.2%}; with each layer set held out of\n")
         f.write(f"// the fit in turn: {held_chosen / held_best - 1:.2%}.\n")
