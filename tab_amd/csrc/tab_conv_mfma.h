@@ -641,7 +641,7 @@ hipError_t launch_mfma_regs(const ConvArgs &a, hipStream_t stream);
 // 8 = 64x64 with K split over the four waves (each wave 2x2 MFMA tiles over a quarter of every chunk), 9 = 128x128 with K
 // split over two pairs of waves (each wave 2x4 MFMA tiles over half of every chunk); both need an even number of words per
 // pixel and otherwise run as shapes 2 and 0, 10 = 128x128 tiles for the whole rounds of the chip and 64x64 split-K quarters for
-// the rest of the last round (words per pixel in fours; otherwise shape 0)
+// the rest of the last round (an even number of words per pixel; otherwise shape 0)
 template <int TYPE>
 hipError_t launch_mfma_type(const ConvArgs &a, int shape, hipStream_t stream)
 {
@@ -652,7 +652,7 @@ hipError_t launch_mfma_type(const ConvArgs &a, int shape, hipStream_t stream)
         if (shape == 7) return hipErrorInvalidValue;
     }
     if (shape == 10) {
-        if (a.PC % 4 == 0) return launch_mfma_tail<TYPE>(a, stream);
+        if (a.PC % 2 == 0) return launch_mfma_tail<TYPE>(a, stream);
         shape = 0;
     }
     if (shape == 8 && a.PC % 2 != 0) shape = 2;

@@ -426,21 +426,22 @@ __attribute__((amdgpu_waves_per_eu(mfma_waves_per_eu(KS > 1 ? 1 : WM, TM, TN, 4 
 
 // Mixed launch for grids of a few rounds of the chip: a launch lasts as long as its busiest CU, and with T tiles on C CUs that
 // is ceil(T / C) tiles although the mean is T / C (392 tiles of 128x128 on 256 CUs: two against 1.53; 784: four against 3.06).
-// Here the first floor(T / C) * C workgroups take whole 128x128 tiles (four MFMA tiles a wave, chunks of four words) and the
-// remaining tiles are cut into four 64x64 quarters each, run by the split-K body (the large tile's ratio of expansions to
-// MFMAs): the last, partial round is dealt out in quarters, so the busiest CU carries at most a quarter tile more than the
-// others.  Workgroups are dispatched in index order, whole tiles first.  Needs words per pixel in fours (PC % 4 == 0).
-template <int TYPE, int ARUN, bool PACKED>
+// Here the first floor(T / C) * C workgroups take whole 128x128 tiles (four MFMA tiles a wave, chunks of KCH words as the plain
+// 128x128 launch would take them) and the remaining tiles are cut into four 64x64 quarters each, run by the split-K body (the
+// large tile's ratio of expansions to MFMAs): the last, partial round is dealt out in quarters, so the busiest CU carries at
+// most a quarter tile more than the others.  Workgroups are dispatched in index order, whole tiles first.  Needs an even
+// number of words per pixel.
+template <int TYPE, int KCH, int ARUN, bool PACKED>
 __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(4))) void conv_mfma_tail(const ConvArgs p)
 {
-    constexpr int BIG = conv_mfma_direct_lds_dwords<TYPE, 2, 2, 2, 2, 4, 1>(), SMALL = conv_mfma_direct_lds_dwords<TYPE, 1, 1, 2, 2, 8, 4>();
+    constexpr int BIG = conv_mfma_direct_lds_dwords<TYPE, 2, 2, 2, 2, KCH, 1>(), SMALL = conv_mfma_direct_lds_dwords<TYPE, 1, 1, 2, 2, 8, 4>();
     __shared__ __attribute__((aligned(16))) uint32_t lds[BIG > SMALL ? BIG : SMALL];
     const uint32_t b = blockIdx.x;
     if (b < (uint32_t)p.tail_big) {  // uniform over the workgroup
         // XCD-aware order over the whole tiles, as in tile_of_workgroup
         const uint32_t logical = b < 8u * (uint32_t)p.xcd_share ? (b & 7u) * (uint32_t)p.xcd_share + (b >> 3) : b;
         const int tile_m = (int)div32(logical, p.div_filter_tiles);
-        conv_mfma_direct_tile<TYPE, 2, 2, 2, 2, 4, PACKED, 1, 0>(p, lds, tile_m, (int)logical - tile_m * p.filter_tiles);
+        conv_mfma_direct_tile<TYPE, 2, 2, 2, 2, KCH, PACKED, 1, 0>(p, lds, tile_m, (int)logical - tile_m * p.filter_tiles);
     } else {
         const uint32_t j = b - (uint32_t)p.tail_big, t = (uint32_t)p.tail_big + (j >> 2), q = j & 3u;
         const int big_m = (int)div32(t, p.div_filter_tiles), big_n = (int)t - big_m * p.filter_tiles;
@@ -450,22 +451,24 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(4)
     }
 }
 
-template <int TYPE, int ARUN>
+template <int TYPE, int KCH, int ARUN>
 hipError_t launch_mfma_tail_run(ConvArgs a, long blocks, hipStream_t stream)
 {
+    a.kcw = KCH;
+    a.nchunks = a.G / KCH;
     if (a.qy != nullptr) {
         if constexpr (TYPE <= 3)
-            conv_mfma_tail<TYPE, ARUN, true><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
+            conv_mfma_tail<TYPE, KCH, ARUN, true><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
         else
             return hipErrorInvalidValue;  // no packed output for types 4 and 5
     } else {
-        conv_mfma_tail<TYPE, ARUN, false><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
+        conv_mfma_tail<TYPE, KCH, ARUN, false><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
     }
     return hipGetLastError();
 }
 
-// False when the layer does not fit the mixed launch (words per pixel not in fours).
-inline bool mfma_tail_supported(const ConvArgs &a) { return a.PC % 4 == 0; }
+// False when the layer does not fit the mixed launch (an odd number of words per pixel).
+inline bool mfma_tail_supported(const ConvArgs &a) { return a.PC % 2 == 0; }
 
 template <int TYPE>
 hipError_t launch_mfma_tail(ConvArgs a, hipStream_t stream)
@@ -476,17 +479,29 @@ hipError_t launch_mfma_tail(ConvArgs a, hipStream_t stream)
     const long whole = tiles / round * round;
     const long blocks = whole + 4 * (tiles - whole);
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
-    a.kcw = 4;
-    a.nchunks = a.G / 4;
     a.tiles_m = (a.M + 127) / 128;
     a.tiles_n = 0;
     a.tail_big = (int)whole;
     a.filter_tiles = (int)filter_tiles;
     a.div_filter_tiles = make_div32((uint32_t)filter_tiles);
     a.xcd_share = whole >= 64 ? (int)(whole / 8) : 0;
-    // granules of an activation pixel: runs of four where the pixel has them, else of two (one-plane operands on 256 channels)
-    if (a.PC * Planes<TYPE>::A / 2 % 4 == 0) return launch_mfma_tail_run<TYPE, 4>(a, blocks, stream);
-    return launch_mfma_tail_run<TYPE, 2>(a, blocks, stream);
+    // The whole tiles' chunk as the plain 128x128 launch picks it (launch_mfma_shape): four words inside a tap, else six words
+    // across taps for the operand pairs that leave LDS for four workgroups a CU, else two.  The quarters' run of activation
+    // granules from the granules of a pixel, as launch_mfma_split picks it.
+    constexpr int APL = Planes<TYPE>::A;
+    const int granules_per_pixel = a.PC * APL / 2;
+    if (a.PC % 4 == 0) {
+        if (granules_per_pixel % 4 == 0) return launch_mfma_tail_run<TYPE, 4, 4>(a, blocks, stream);
+        return launch_mfma_tail_run<TYPE, 4, 2>(a, blocks, stream);
+    }
+    if constexpr (APL + Planes<TYPE>::B <= 3) {
+        if (a.G % 6 == 0) {
+            if constexpr (APL == 2) return launch_mfma_tail_run<TYPE, 6, 2>(a, blocks, stream);
+            return launch_mfma_tail_run<TYPE, 6, 1>(a, blocks, stream);
+        }
+    }
+    if constexpr (APL == 2) return launch_mfma_tail_run<TYPE, 2, 2>(a, blocks, stream);
+    return launch_mfma_tail_run<TYPE, 2, 1>(a, blocks, stream);
 }
 
 template <int TYPE, int WM, int WN, int TM, int TN, int KCH, int KS, int ARUN>

@@ -35,6 +35,9 @@ GEOMETRIES = [
     (1, 28, 28, 256, 64, 1, 1, 0, 0, 1, 1),              # 7 x 1, four words of K: one zero-padded chunk of eight in the quarters
     (7, 8, 8, 256, 384, 3, 3, 1, 0, 1, 1),               # 3 x 3
     (2, 12, 12, 768, 96, 2, 2, 0, 1, 1, 1),              # twelve words per pixel, 2x2 taps
+    (3, 16, 16, 128, 256, 3, 3, 1, 1, 1, 1),             # two words per pixel: the whole tiles take chunks of six words across taps
+    (2, 10, 10, 384, 130, 3, 3, 1, 1, 1, 1),             # six words per pixel
+    (2, 9, 9, 128, 70, 2, 2, 0, 0, 1, 1),                # two words per pixel, K = 8 words: whole tiles in chunks of two
 ]
 
 
