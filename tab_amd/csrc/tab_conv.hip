@@ -427,10 +427,12 @@ int conv_mfma_shape(int conv_type, const ConvArgs &a, float *cost_us)
         const long tiles = (long)((a.M + bm - 1) / bm) * ((a.KN + bn - 1) / bn);
         float cost = 0.f, floor_us;
         if (shape == 10) {
-            // the mixed launch: whole tiles on every CU, then quarter tiles; a candidate where it has both and K is more than
-            // 18 words (with a short K the launch is bound by writing Y, whatever the balance of its last round)
+            // the mixed launch: whole tiles on every CU, then quarter tiles; a candidate where it has both and K words x bit
+            // planes of the two operands exceed 36 (below that the launch is bound by writing Y, whatever the balance of its
+            // last round)
             const long whole = tiles / cus, quarters = (4 * (tiles % cus) + cus - 1) / cus;
-            if (a.G <= 18 || whole == 0 || quarters == 0) continue;  // (an odd number of words per pixel: excluded above)
+            const int planes = type == 0 ? 4 : (type == 3 ? 2 : 3);
+            if (a.G * planes <= 36 || whole == 0 || quarters == 0) continue;  // (an odd number of words per pixel: excluded above)
             const float f[kConvShapeFeatures] = {(float)a.G * (float)whole, (float)a.G * (float)quarters, (float)quarters, (float)whole, y_mb, y_mb,
                                                  1.f, 1.f, 0.f};
             for (int k = 0; k < kConvShapeFeatures; k++) cost += kConvShapeCost[type][i][k] * f[k];

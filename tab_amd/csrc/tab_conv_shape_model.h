@@ -1,12 +1,12 @@
 // Written by tab_amd/tuning/fit_conv_shape_model.py from tab_amd/tuning/conv_shape_training_timings.txt: do not edit.
-// Fitted 2026-11-25 on the kernels of commit 3826976 (and the working tree on top of it).
+// Fitted 2026-11-25 on the kernels of commit d089cb0 (and the working tree on top of it).
 // Cost model of the matrix-core workgroup shapes: predicted duration (us) = kConvShapeCost[type][i] . f for the shape
 // kConvShapeIds[i], f = {G*n, G*rounds, rounds, n, Y, Y*busy, busy, 1, Y*[G <= 9]} (n = tiles on the busiest CU,
 // rounds = refills of that CU, Y = megabytes of output, busy = share of the CUs with work; shape 10, the mixed launch:
 // {G*whole, G*quarters, quarters, whole, Y, Y, 1, 1, Y*[G <= 9]}, whole tiles per CU and quarter tiles after them).  Non-negative least squares:
 // every feature and every coefficient is >= 0, so a prediction is positive and monotone for any geometry.  Regret of the
-// choice against the best measured shape over the 280 fitted cases: 1.22%; with each layer set held out of
-// the fit in turn: 1.79%.
+// choice against the best measured shape over the 280 fitted cases: 1.29%; with each layer set held out of
+// the fit in turn: 1.86%.
 #pragma once
 
 namespace tab {
@@ -27,7 +27,7 @@ constexpr float kConvShapeCost[4][kConvShapes][kConvShapeFeatures] = {
         {0.128618f, 0.118425f, 0.0f, 0.0f, 0.0723173f, 0.0463867f, 0.743713f, 4.19554f, 0.0173782f},
         {0.0251956f, 0.0396773f, 0.0f, 0.670934f, 0.0254314f, 0.0f, 0.734947f, 3.29611f, 0.0f},
         {0.0628066f, 0.0892484f, 0.826519f, 0.0390676f, 0.112093f, 0.0f, 0.0317503f, 4.3067f, 0.0159801f},
-        {0.129589f, 0.0308505f, 0.991094f, 0.0f, 0.0823405f, 0.0f, 2.92355f, 0.0f, 0.0f},
+        {0.131062f, 0.0280487f, 1.21232f, 0.0f, 0.0760424f, 0.0f, 2.93196f, 0.0f, 0.0f},
     },
     {
         {0.0865426f, 0.0693587f, 0.0f, 0.0f, 0.0579624f, 0.0f, 1.82022f, 2.9411f, 0.0648396f},
@@ -39,7 +39,7 @@ constexpr float kConvShapeCost[4][kConvShapes][kConvShapeFeatures] = {
         {0.121266f, 0.0798943f, 0.0f, 0.0f, 0.0885932f, 0.0317639f, 0.564441f, 3.91746f, 0.0156865f},
         {0.022049f, 0.0348356f, 0.0f, 0.768156f, 0.0f, 0.0f, 0.620039f, 3.04518f, 0.0f},
         {0.0613883f, 0.0738368f, 1.12291f, 0.0f, 0.0950171f, 0.0f, 0.305162f, 3.77746f, 0.0184637f},
-        {0.109751f, 0.0323941f, 0.499123f, 0.0f, 0.0806325f, 0.0f, 3.46044f, 0.0f, 0.0f},
+        {0.111417f, 0.0296573f, 0.654945f, 0.0f, 0.0718793f, 0.0f, 3.698f, 0.0f, 0.0f},
     },
     {
         {0.0921608f, 0.0695768f, 0.0f, 0.0f, 0.0494465f, 0.0f, 1.69354f, 3.09981f, 0.0724312f},
@@ -51,7 +51,7 @@ constexpr float kConvShapeCost[4][kConvShapes][kConvShapeFeatures] = {
         {0.138187f, 0.0742667f, 0.0f, 0.0f, 0.0964049f, 0.0304895f, 0.290869f, 4.27502f, 0.00752971f},
         {0.0234524f, 0.0278454f, 0.0f, 0.699996f, 0.0246471f, 0.0f, 0.61602f, 3.03661f, 0.00496521f},
         {0.0751333f, 0.0522657f, 0.737833f, 0.0181711f, 0.116729f, 0.0f, 0.0f, 4.44661f, 0.00639848f},
-        {0.108259f, 0.0316604f, 0.775299f, 0.0f, 0.0867138f, 0.0f, 3.18729f, 0.0f, 0.0f},
+        {0.110379f, 0.0315015f, 0.678581f, 0.0f, 0.0755007f, 0.0f, 3.64185f, 0.0f, 0.0f},
     },
     {
         {0.070951f, 0.0583979f, 0.0f, 0.0f, 0.07163f, 0.0f, 1.72993f, 2.88768f, 0.0573304f},

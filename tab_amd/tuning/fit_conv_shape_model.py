@@ -15,9 +15,10 @@ The mixed launch (shape 10: 128x128 tiles for the whole rounds of the chip, 64x6
     f = [G*whole, G*quarters, quarters, whole, Y, Y, 1, 1, Y*[G <= 9]]
     whole    = floor(tiles / 256)                    whole tiles on every CU
     quarters = ceil(4 * (tiles mod 256) / 256)       quarter tiles on the busiest CU after them
-and is a candidate where both are positive, the words per pixel are even in number and K is more than 18 words (the MFMA
-work per byte of Y grows with K alone; with a short K the launch is bound by writing Y and gains nothing from a better
-balanced last round: N=256 28x28x128->256 3x3 stride 2, K = 18 words, 16.1 us mixed or plain against 13.9 with 128x64 tiles).
+and is a candidate where both are positive, the words per pixel are even in number and K words x bit planes of the two
+operands exceed 36 (the work per byte of Y grows with K and with the planes to expand alone; below that the launch is bound
+by writing Y and gains nothing from a better balanced last round: BNN N=256 28x28x128->256 3x3 stride 2, K = 18 words,
+16.1 us mixed or plain against 13.9 with 128x64 tiles, where the ternary types gain 6-10 %).
 fitted by NON-NEGATIVE least squares on relative error (the N=16 set weighted threefold): every feature is non-negative and
 so is every coefficient, hence a predicted duration is positive and grows with K, with the tiles on the busiest CU and
 with Y for every geometry, inside the fitted range or far outside it (an unconstrained fit had coefficients of both signs,
@@ -38,6 +39,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 SHAPES = {0: (128, 128, 4), 1: (128, 64, 6), 2: (64, 64, 8), 3: (32, 32, 4), 4: (256, 64, 4), 5: (256, 128, 2), 6: (128, 256, 2),
           8: (64, 64, 4), 9: (128, 128, 2), 10: (128, 128, 4)}
 MIXED = 10
+PLANES = {0: 4, 1: 3, 2: 3, 3: 2}  # bit planes of activation + weight operand, per type
 IDS = sorted(SHAPES)
 NFEAT = 9
 
@@ -66,7 +68,7 @@ def mixed_rounds(r):
 
 def eligible(r, s):
     # (the split-K shapes need an even number of words per pixel; otherwise they run as shapes 2 and 0)
-    if s == MIXED and (r["G"] <= 18 or 0 in mixed_rounds(r)):
+    if s == MIXED and (r["G"] * PLANES[r["type"]] <= 36 or 0 in mixed_rounds(r)):
         return False
     return SHAPES[s][1] < 2 * (-(-r["KN"] // 64) * 64) and s in r["times"] and not (s >= 8 and r["PC"] % 2)
 

@@ -41,7 +41,7 @@ def test_every_choice_is_legal_and_priced_positive():
         assert bn < 2 * ((KN + 63) // 64 * 64), what          # a filter tile under twice the filters
         assert not (packed and shape == 3), what              # packed output needs 64-filter tiles
         assert not (shape >= 8 and PC % 2), what              # split-K shapes: an even number of words per pixel
-        assert not (shape == 10 and (G <= 18 or M * KN < 128 * 128 * 2)), what   # the mixed launch: a long K, more than a round
+        assert not (shape == 10 and (G <= 9 or M * KN < 128 * 128 * 2)), what   # the mixed launch: a long K, more than a round
         assert math.isfinite(cost) and cost > 0.9, what       # never below a launch
 
 
