@@ -217,8 +217,9 @@ int tab_conv2d_packed_out(const int64_t *dev_QX, const int64_t *dev_QW, const in
  *                      9: 128x128 with K split over four / two groups of waves inside the workgroup (an
  *                      even number of words per pixel; otherwise tiles 2 and 0), 10: 128x128 for the
  *                      whole rounds of the chip and 64x64 quarters, K split over the waves, for the rest
- *                      of the last round (an even number of words per pixel; otherwise tile 0); -1: picked
- *                      from the shape
+ *                      of the last round (an even number of words per pixel; otherwise tile 0), 11: the
+ *                      same with whole tiles of 128x256 (words per pixel in fours; otherwise tile 6); -1:
+ *                      picked from the shape
  *   TAB_CONV_POPCOUNT  the reference's xor/and + popcount formulation on the vector ALU;
  *                      tile 0: big, 1: medium, 2: small; -1: picked from the shape
  *                      (types 4 and 5 exist on the matrix cores only and ignore this choice)

@@ -337,7 +337,7 @@ CONV_AUTO, CONV_MATRIX, CONV_POPCOUNT = 0, 1, 2
 
 
 def set_conv_kernel(kernel=CONV_AUTO, tile=-1):
-    """Pick the conv kernel (process-wide): CONV_AUTO, CONV_MATRIX (tile 0..10 or -1) or
+    """Pick the conv kernel (process-wide): CONV_AUTO, CONV_MATRIX (tile 0..11 or -1) or
     CONV_POPCOUNT (tile 0..2 or -1).  Every choice gives bit-identical outputs."""
     _capi.check(_lib, _lib.tab_set_conv_kernel(int(kernel), int(tile)))
 

@@ -113,7 +113,7 @@ int tab_set_conv_kernel(int kernel, int tile)
 {
     static const int popcount_tm[4] = {7, 8, 4, 2};  // 7: the popcount kernel's own choice
     if (kernel == TAB_CONV_AUTO && tile == -1) tab::force_conv_tile(0, 0);
-    else if (kernel == TAB_CONV_MATRIX && tile >= -1 && tile <= 10) tab::force_conv_tile(9, tile);
+    else if (kernel == TAB_CONV_MATRIX && tile >= -1 && tile <= 11) tab::force_conv_tile(9, tile);
     else if (kernel == TAB_CONV_POPCOUNT && tile >= -1 && tile <= 2) tab::force_conv_tile(popcount_tm[tile + 1], 0);
     else return fail(TAB_ERR_BAD_ARGUMENT, "no conv kernel %d with tile %d", kernel, tile);
     return TAB_OK;

@@ -426,17 +426,19 @@ int conv_mfma_shape(int conv_type, const ConvArgs &a, float *cost_us)
         if (shape >= 8 && a.PC % 2 != 0) continue;          // the split-K shapes move whole pairs of words inside a tap
         const long tiles = (long)((a.M + bm - 1) / bm) * ((a.KN + bn - 1) / bn);
         float cost = 0.f, floor_us;
-        if (shape == 10) {
-            // the mixed launch: whole tiles on every CU, then quarter tiles; a candidate where it has both and K words x bit
-            // planes of the two operands exceed 36 (below that the launch is bound by writing Y, whatever the balance of its
-            // last round)
-            const long whole = tiles / cus, quarters = (4 * (tiles % cus) + cus - 1) / cus;
+        if (shape == 10 || shape == 11) {
+            // the mixed launches: whole tiles on every CU, then 64x64 quarter tiles (four to a 128x128 tile, eight to a
+            // 128x256 one); candidates where they have both and K words x bit planes of the two operands exceed 36 (below
+            // that the launch is bound by writing Y, whatever the balance of its last round)
+            const long pieces = bm / 64 * (bn / 64);
+            const long whole = tiles / cus, quarters = (pieces * (tiles % cus) + cus - 1) / cus;
             const int planes = type == 0 ? 4 : (type == 3 ? 2 : 3);
             if (a.G * planes <= 36 || whole == 0 || quarters == 0) continue;  // (an odd number of words per pixel: excluded above)
+            if (shape == 11 && a.PC % 4 != 0) continue;                       // the 128x256 tiles take four-word chunks inside a tap
             const float f[kConvShapeFeatures] = {(float)a.G * (float)whole, (float)a.G * (float)quarters, (float)quarters, (float)whole, y_mb, y_mb,
                                                  1.f, 1.f, 0.f};
             for (int k = 0; k < kConvShapeFeatures; k++) cost += kConvShapeCost[type][i][k] * f[k];
-            floor_us = 1.f + (float)(16 * whole + 4 * quarters) * (float)a.G * (32.f / 4.f / 2400.f);
+            floor_us = 1.f + (float)(4 * pieces * whole + 4 * quarters) * (float)a.G * (32.f / 4.f / 2400.f);
         } else {
             const float n = (float)((tiles + cus - 1) / cus), rounds = (float)(((tiles + cus - 1) / cus + held - 1) / held);
             const float busy = tiles >= cus ? 1.f : (float)tiles / (float)cus;
@@ -463,7 +465,7 @@ hipError_t launch_conv(int type, const ConvArgs &args, hipStream_t stream)
     const int force_tm = forced.tm, force_ng = forced.ng;
     if (args.qy != nullptr) {  // packed output exists in the matrix-core kernel's 64-wide shapes only
         if (!conv_mfma_exact(args)) return hipErrorInvalidValue;
-        const int shape = (force_tm == 9 && force_ng >= 0 && force_ng != 3 && force_ng <= 10) ? force_ng : conv_mfma_shape(type, args);
+        const int shape = (force_tm == 9 && force_ng >= 0 && force_ng != 3 && force_ng <= 11) ? force_ng : conv_mfma_shape(type, args);
         return launch_conv_mfma(type, args, shape, stream);
     }
     if (force_tm == 9) return launch_conv_mfma(type, args, force_ng < 0 ? conv_mfma_shape(type, args) : force_ng, stream);

@@ -589,6 +589,8 @@ template <int TYPE, int WM, int WN, int TM, int TN, int KS, int WORDS>
 hipError_t launch_mfma_split(const ConvArgs &a, hipStream_t stream);
 template <int TYPE>
 hipError_t launch_mfma_tail(ConvArgs a, hipStream_t stream);
+template <int TYPE>
+hipError_t launch_mfma_tail_wide(ConvArgs a, hipStream_t stream);
 
 template <int TYPE, int WM, int WN, int TM, int TN, int KCH, int KS = 1>
 hipError_t launch_mfma_intap(const ConvArgs &a, hipStream_t stream)
@@ -641,7 +643,8 @@ hipError_t launch_mfma_regs(const ConvArgs &a, hipStream_t stream);
 // 8 = 64x64 with K split over the four waves (each wave 2x2 MFMA tiles over a quarter of every chunk), 9 = 128x128 with K
 // split over two pairs of waves (each wave 2x4 MFMA tiles over half of every chunk); both need an even number of words per
 // pixel and otherwise run as shapes 2 and 0, 10 = 128x128 tiles for the whole rounds of the chip and 64x64 split-K quarters for
-// the rest of the last round (an even number of words per pixel; otherwise shape 0)
+// the rest of the last round (an even number of words per pixel; otherwise shape 0), 11 = the same with whole tiles of 128x256
+// (words per pixel in fours; otherwise shape 6)
 template <int TYPE>
 hipError_t launch_mfma_type(const ConvArgs &a, int shape, hipStream_t stream)
 {
@@ -650,6 +653,10 @@ hipError_t launch_mfma_type(const ConvArgs &a, int shape, hipStream_t stream)
             if (a.G <= 9) return launch_mfma_regs<TYPE>(a, stream);
         shape = conv_mfma_shape(TYPE, a);
         if (shape == 7) return hipErrorInvalidValue;
+    }
+    if (shape == 11) {
+        if (a.PC % 4 == 0) return launch_mfma_tail_wide<TYPE>(a, stream);
+        shape = 6;
     }
     if (shape == 10) {
         if (a.PC % 2 == 0) return launch_mfma_tail<TYPE>(a, stream);

@@ -431,44 +431,67 @@ __attribute__((amdgpu_waves_per_eu(mfma_waves_per_eu(KS > 1 ? 1 : WM, TM, TN, 4 
 // large tile's ratio of expansions to MFMAs): the last, partial round is dealt out in quarters, so the busiest CU carries at
 // most a quarter tile more than the others.  Workgroups are dispatched in index order, whole tiles first.  Needs an even
 // number of words per pixel.
-template <int TYPE, int KCH, int ARUN, bool PACKED>
-__global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(4))) void conv_mfma_tail(const ConvArgs p)
+// TNB = 4: the whole tiles are 128x256 (eight MFMA tiles a wave, the pipelined loop, two workgroups a CU) and a remaining tile
+// makes eight quarters.
+template <int TYPE, int KCH, int ARUN, bool PACKED, int TNB = 2>
+__global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TNB == 4 ? 2 : 4))) void conv_mfma_tail(const ConvArgs p)
 {
-    constexpr int BIG = conv_mfma_direct_lds_dwords<TYPE, 2, 2, 2, 2, KCH, 1>(), SMALL = conv_mfma_direct_lds_dwords<TYPE, 1, 1, 2, 2, 8, 4>();
+    constexpr int BIG = conv_mfma_direct_lds_dwords<TYPE, 2, 2, 2, TNB, KCH, 1>(), SMALL = conv_mfma_direct_lds_dwords<TYPE, 1, 1, 2, 2, 8, 4>();
     __shared__ __attribute__((aligned(16))) uint32_t lds[BIG > SMALL ? BIG : SMALL];
     const uint32_t b = blockIdx.x;
     if (b < (uint32_t)p.tail_big) {  // uniform over the workgroup
         // XCD-aware order over the whole tiles, as in tile_of_workgroup
         const uint32_t logical = b < 8u * (uint32_t)p.xcd_share ? (b & 7u) * (uint32_t)p.xcd_share + (b >> 3) : b;
         const int tile_m = (int)div32(logical, p.div_filter_tiles);
-        conv_mfma_direct_tile<TYPE, 2, 2, 2, 2, KCH, PACKED, 1, 0>(p, lds, tile_m, (int)logical - tile_m * p.filter_tiles);
+        conv_mfma_direct_tile<TYPE, 2, 2, 2, TNB, KCH, PACKED, 1, 0>(p, lds, tile_m, (int)logical - tile_m * p.filter_tiles);
     } else {
-        const uint32_t j = b - (uint32_t)p.tail_big, t = (uint32_t)p.tail_big + (j >> 2), q = j & 3u;
+        constexpr uint32_t PIECES = 2 * TNB;  // 64x64 quarters of a whole tile
+        const uint32_t j = b - (uint32_t)p.tail_big, t = (uint32_t)p.tail_big + j / PIECES, q = j % PIECES;
         const int big_m = (int)div32(t, p.div_filter_tiles), big_n = (int)t - big_m * p.filter_tiles;
-        const int tile_m = 2 * big_m + (int)(q & 1u), tile_n = 2 * big_n + (int)(q >> 1);
+        const int tile_m = 2 * big_m + (int)(q & 1u), tile_n = TNB * big_n + (int)(q >> 1);
         if (tile_m * 64 >= p.M || tile_n * 64 >= p.KN) return;  // a quarter wholly past the edge of Y
         conv_mfma_direct_tile<TYPE, 1, 1, 2, 2, 8, PACKED, 4, ARUN>(p, lds, tile_m, tile_n);
     }
 }
 
-template <int TYPE, int KCH, int ARUN>
+template <int TYPE, int KCH, int ARUN, int TNB = 2>
 hipError_t launch_mfma_tail_run(ConvArgs a, long blocks, hipStream_t stream)
 {
     a.kcw = KCH;
     a.nchunks = a.G / KCH;
     if (a.qy != nullptr) {
         if constexpr (TYPE <= 3)
-            conv_mfma_tail<TYPE, KCH, ARUN, true><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
+            conv_mfma_tail<TYPE, KCH, ARUN, true, TNB><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
         else
             return hipErrorInvalidValue;  // no packed output for types 4 and 5
     } else {
-        conv_mfma_tail<TYPE, KCH, ARUN, false><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
+        conv_mfma_tail<TYPE, KCH, ARUN, false, TNB><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
     }
     return hipGetLastError();
 }
 
 // False when the layer does not fit the mixed launch (an odd number of words per pixel).
 inline bool mfma_tail_supported(const ConvArgs &a) { return a.PC % 2 == 0; }
+
+// Whole tiles of 128x256 (words per pixel in fours).
+template <int TYPE>
+hipError_t launch_mfma_tail_wide(ConvArgs a, hipStream_t stream)
+{
+    if (a.PC % 4 != 0) return hipErrorInvalidValue;
+    const long filter_tiles = (a.KN + 255) / 256, tiles = (long)((a.M + 127) / 128) * filter_tiles;
+    const long round = tail_round();
+    const long whole = tiles / round * round;
+    const long blocks = whole + 8 * (tiles - whole);
+    if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
+    a.tiles_m = (a.M + 127) / 128;
+    a.tiles_n = 0;
+    a.tail_big = (int)whole;
+    a.filter_tiles = (int)filter_tiles;
+    a.div_filter_tiles = make_div32((uint32_t)filter_tiles);
+    a.xcd_share = whole >= 64 ? (int)(whole / 8) : 0;
+    if (a.PC * Planes<TYPE>::A / 2 % 4 == 0) return launch_mfma_tail_run<TYPE, 4, 4, 4>(a, blocks, stream);
+    return launch_mfma_tail_run<TYPE, 4, 2, 4>(a, blocks, stream);
+}
 
 template <int TYPE>
 hipError_t launch_mfma_tail(ConvArgs a, hipStream_t stream)

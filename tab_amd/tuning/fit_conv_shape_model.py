@@ -11,11 +11,12 @@ Model, per (type, shape): duration ~ c . f with the features
     busy   = min(1, tiles / 256)                     share of the CUs that have work at all
     G      = KH*KW*PC words of K, Y = 4*M*KN bytes / 1e6; the last feature gives the layers whose loop is a handful of
              MFMAs (C = 64 with 3x3, 1x1) their own price per byte of Y: their launches are the epilogue
-The mixed launch (shape 10: 128x128 tiles for the whole rounds of the chip, 64x64 split-K quarters for the rest) has
+The mixed launches (shape 10: 128x128 tiles for the whole rounds of the chip, 64x64 split-K quarters for the rest; shape 11:
+the same with 128x256 tiles, eight quarters to a tile, words per pixel in fours) have
     f = [G*whole, G*quarters, quarters, whole, Y, Y, 1, 1, Y*[G <= 9]]
     whole    = floor(tiles / 256)                    whole tiles on every CU
     quarters = ceil(4 * (tiles mod 256) / 256)       quarter tiles on the busiest CU after them
-and is a candidate where both are positive, the words per pixel are even in number and K words x bit planes of the two
+and are candidates where both are positive, the words per pixel are even in number and K words x bit planes of the two
 operands exceed 36 (the work per byte of Y grows with K and with the planes to expand alone; below that the launch is bound
 by writing Y and gains nothing from a better balanced last round: BNN N=256 28x28x128->256 3x3 stride 2, K = 18 words,
 16.1 us mixed or plain against 13.9 with 128x64 tiles, where the ternary types gain 6-10 %).
@@ -37,8 +38,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 # shape id -> rows x filters of the workgroup tile, workgroups a CU holds (the occupancy the compiler reports for the
 # shape's kernels with four-word chunks: registers, or LDS where that is the tighter limit)
 SHAPES = {0: (128, 128, 4), 1: (128, 64, 6), 2: (64, 64, 8), 3: (32, 32, 4), 4: (256, 64, 4), 5: (256, 128, 2), 6: (128, 256, 2),
-          8: (64, 64, 4), 9: (128, 128, 2), 10: (128, 128, 4)}
-MIXED = 10
+          8: (64, 64, 4), 9: (128, 128, 2), 10: (128, 128, 4), 11: (128, 256, 2)}
+MIXED = (10, 11)
 PLANES = {0: 4, 1: 3, 2: 3, 3: 2}  # bit planes of activation + weight operand, per type
 IDS = sorted(SHAPES)
 NFEAT = 9
@@ -61,14 +62,15 @@ def parse(path):
     return rows
 
 
-def mixed_rounds(r):
-    tiles = -(-r["M"] // 128) * -(-r["KN"] // 128)
-    return tiles // 256, -(-4 * (tiles % 256) // 256)
+def mixed_rounds(r, s):
+    BM, BN, _ = SHAPES[s]
+    tiles = -(-r["M"] // BM) * -(-r["KN"] // BN)
+    return tiles // 256, -(-(BM // 64 * (BN // 64)) * (tiles % 256) // 256)
 
 
 def eligible(r, s):
     # (the split-K shapes need an even number of words per pixel; otherwise they run as shapes 2 and 0)
-    if s == MIXED and (r["G"] * PLANES[r["type"]] <= 36 or 0 in mixed_rounds(r)):
+    if s in MIXED and (r["G"] * PLANES[r["type"]] <= 36 or 0 in mixed_rounds(r, s) or (s == 11 and r["PC"] % 4)):
         return False
     return SHAPES[s][1] < 2 * (-(-r["KN"] // 64) * 64) and s in r["times"] and not (s >= 8 and r["PC"] % 2)
 
@@ -76,8 +78,8 @@ def eligible(r, s):
 def features(r, s):
     BM, BN, held = SHAPES[s]
     Y = r["M"] * r["KN"] * 4e-6
-    if s == MIXED:
-        whole, quarters = mixed_rounds(r)
+    if s in MIXED:
+        whole, quarters = mixed_rounds(r, s)
         return [r["G"] * whole, r["G"] * quarters, quarters, whole, Y, Y, 1.0, 1.0, Y if r["G"] <= 9 else 0.0]
     tiles = -(-r["M"] // BM) * -(-r["KN"] // BN)
     n = -(-tiles // 256)
@@ -147,7 +149,7 @@ def main():
         f.write(f"// Fitted {datetime.date.today().isoformat()} on the kernels of commit {commit} (and the working tree on top of it).\n")
         f.write("// Cost model of the matrix-core workgroup shapes: predicted duration (us) = kConvShapeCost[type][i] . f for the shape\n")
         f.write("// kConvShapeIds[i], f = {G*n, G*rounds, rounds, n, Y, Y*busy, busy, 1, Y*[G <= 9]} (n = tiles on the busiest CU,\n")
-        f.write("// rounds = refills of that CU, Y = megabytes of output, busy = share of the CUs with work; shape 10, the mixed launch:\n")
+        f.write("// rounds = refills of that CU, Y = megabytes of output, busy = share of the CUs with work; shapes 10 and 11, the mixed launches:\n")
         f.write("// {G*whole, G*quarters, quarters, whole, Y, Y, 1, 1, Y*[G <= 9]}, whole tiles per CU and quarter tiles after them).  Non-negative least squares:\n")
         f.write("// every feature and every coefficient is >= 0, so a prediction is positive and monotone for any geometry.  Regret of the\n")
         f.write(f"// choice against the best measured shape over the {len(rows)} fitted cases: {total:.2%}; with each layer set held out of\n")

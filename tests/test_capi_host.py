@@ -132,7 +132,7 @@ def test_conv2d_launches_names_the_one_launch_cases():
 def test_set_conv_kernel_validates_without_a_gpu():
     lib = _capi.load()
     try:
-        for kernel, tile, ok in [(0, -1, True), (1, -1, True), (1, 6, True), (1, 7, True), (1, 10, True), (1, 11, False), (2, 2, True), (2, 3, False),
+        for kernel, tile, ok in [(0, -1, True), (1, -1, True), (1, 6, True), (1, 7, True), (1, 11, True), (1, 12, False), (2, 2, True), (2, 3, False),
                                  (0, 0, False), (3, -1, False)]:
             assert (lib.tab_set_conv_kernel(kernel, tile) == 0) == ok, (kernel, tile)
         assert b"no conv kernel" in lib.tab_last_error()

@@ -103,7 +103,7 @@ def test_large_channel_layers(type, case):
     _conv_case(type, *case)
 
 
-KERNEL_VARIANTS = [(tab_amd.CONV_MATRIX, t) for t in range(11)] + [(tab_amd.CONV_POPCOUNT, t) for t in range(3)]
+KERNEL_VARIANTS = [(tab_amd.CONV_MATRIX, t) for t in range(12)] + [(tab_amd.CONV_POPCOUNT, t) for t in range(3)]
 VARIANT_CASES = [
     (2, 9, 6, 70, 5, 3, 3, 1, 0, 1, 2),        # one word per pixel pair: chunks cross taps
     (2, 12, 12, 192, 130, 3, 3, 1, 1, 1, 1),   # PC = 3: odd words per tap
@@ -203,7 +203,7 @@ def test_set_conv_kernel_rejects_unknown():
     with pytest.raises(tab_amd.TabError, match="no conv kernel"):
         tab_amd.set_conv_kernel(5, 0)
     with pytest.raises(tab_amd.TabError, match="no conv kernel"):
-        tab_amd.set_conv_kernel(tab_amd.CONV_MATRIX, 11)
+        tab_amd.set_conv_kernel(tab_amd.CONV_MATRIX, 12)
 
 
 def test_arbitrary_weight_bit_patterns():

@@ -80,7 +80,7 @@ def test_conv2d_from_floats(type, case):
     assert got.shape == want.shape and np.array_equal(got, want), f"max |diff| = {np.abs(got - want).max()}"
 
 
-KERNELS = [(tab_amd.CONV_MATRIX, t) for t in range(11)] + [(tab_amd.CONV_POPCOUNT, -1)]
+KERNELS = [(tab_amd.CONV_MATRIX, t) for t in range(12)] + [(tab_amd.CONV_POPCOUNT, -1)]
 
 
 @pytest.mark.parametrize("type", [4, 5])

@@ -1,5 +1,5 @@
-"""The mixed launch of the matrix-core conv kernel (tab_set_conv_kernel(TAB_CONV_MATRIX, 10)): 128x128 tiles for the whole
-rounds of the chip, 64x64 split-K quarter tiles for the rest of the last round.  A round is the chip's compute units, far
+"""The mixed launches of the matrix-core conv kernel (tab_set_conv_kernel(TAB_CONV_MATRIX, 10 or 11)): 128x128 (10) or 128x256
+(11) tiles for the whole rounds of the chip, 64x64 split-K quarter tiles for the rest of the last round.  A round is the chip's compute units, far
 more tiles than an oracle-sized layer has, so these tests shrink the round through the library's test hook: layers of a few
 tiles then mix whole tiles and quarters, with ragged edges in both.  Bit-exact against the CPU oracle."""
 import ctypes
@@ -16,12 +16,12 @@ from tab_amd import _capi
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture
-def tail_round():
+@pytest.fixture(params=[10, 11])
+def tail_round(request):
     lib = ctypes.CDLL(_capi.LIB_PATH)
     lib.tab_internal_set_tail_round.argtypes = [ctypes.c_int]
     lib.tab_internal_set_tail_round.restype = None
-    tab_amd.set_conv_kernel(tab_amd.CONV_MATRIX, 10)
+    tab_amd.set_conv_kernel(tab_amd.CONV_MATRIX, request.param)
     yield lib.tab_internal_set_tail_round
     lib.tab_internal_set_tail_round(0)
     tab_amd.set_conv_kernel(tab_amd.CONV_AUTO, -1)
@@ -33,7 +33,8 @@ GEOMETRIES = [
     (3, 13, 11, 250, 200, 3, 3, 1, 1, 1, 1),             # 4 x 2, rows, filters and channels ragged
     (5, 9, 9, 512, 130, 3, 3, 1, 1, 2, 2),               # 1 x 2: the second filter tile holds two filters, its second quarter column none
     (1, 28, 28, 256, 64, 1, 1, 0, 0, 1, 1),              # 7 x 1, four words of K: one zero-padded chunk of eight in the quarters
-    (7, 8, 8, 256, 384, 3, 3, 1, 0, 1, 1),               # 3 x 3
+    (7, 8, 8, 256, 384, 3, 3, 1, 0, 1, 1),               # 3 x 3 (3 x 2 of 128 x 256, the second half filled)
+    (4, 10, 10, 256, 600, 3, 3, 1, 1, 1, 1),             # 4 x 5 (4 x 3 of 128 x 256: the last filter tile holds 88 filters)
     (2, 12, 12, 768, 96, 2, 2, 0, 1, 1, 1),              # twelve words per pixel, 2x2 taps
     (3, 16, 16, 128, 256, 3, 3, 1, 1, 1, 1),             # two words per pixel: the whole tiles take chunks of six words across taps
     (2, 10, 10, 384, 130, 3, 3, 1, 1, 1, 1),             # six words per pixel

@@ -69,7 +69,7 @@ def test_packed_out(type, case, out_bits):
         _packed_out_case(type, *case, out_bits, kind, seed=type + out_bits)
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 4, 5, 6, 7, 8, 9, 10])
+@pytest.mark.parametrize("tile", [0, 1, 2, 4, 5, 6, 7, 8, 9, 10, 11])
 @pytest.mark.parametrize("type", [0, 1, 2, 3])
 def test_packed_out_every_tile(type, tile, restore_kernel_choice):
     """Every shape packs its output: C = 192 and 256 take the kernel that multiplies with the weights first and packs

@@ -10,7 +10,7 @@ from helpers import act_bits, make_layer, weight_bits
 
 pytestmark = pytest.mark.gpu
 
-VARIANTS = [(tab_amd.CONV_AUTO, -1)] + [(tab_amd.CONV_MATRIX, t) for t in range(11)] + [(tab_amd.CONV_POPCOUNT, t) for t in range(3)]
+VARIANTS = [(tab_amd.CONV_AUTO, -1)] + [(tab_amd.CONV_MATRIX, t) for t in range(12)] + [(tab_amd.CONV_POPCOUNT, t) for t in range(3)]
 
 
 def _random_case(rng):

@@ -7,7 +7,7 @@ import math
 
 from tab_amd import _capi
 
-TILE = {0: (128, 128), 1: (128, 64), 2: (64, 64), 3: (32, 32), 4: (256, 64), 5: (256, 128), 6: (128, 256), 8: (64, 64), 9: (128, 128), 10: (128, 128)}
+TILE = {0: (128, 128), 1: (128, 64), 2: (64, 64), 3: (32, 32), 4: (256, 64), 5: (256, 128), 6: (128, 256), 8: (64, 64), 9: (128, 128), 10: (128, 128), 11: (128, 256)}
 
 
 def _hook():
@@ -41,7 +41,8 @@ def test_every_choice_is_legal_and_priced_positive():
         assert bn < 2 * ((KN + 63) // 64 * 64), what          # a filter tile under twice the filters
         assert not (packed and shape == 3), what              # packed output needs 64-filter tiles
         assert not (shape >= 8 and PC % 2), what              # split-K shapes: an even number of words per pixel
-        assert not (shape == 10 and (G <= 9 or M * KN < 128 * 128 * 2)), what   # the mixed launch: a long K, more than a round
+        assert not (shape in (10, 11) and (G <= 9 or M * KN < 128 * 128 * 2)), what
+        assert not (shape == 11 and PC % 4), what   # the mixed launch: a long K, more than a round
         assert math.isfinite(cost) and cost > 0.9, what       # never below a launch
 
 
