@@ -92,10 +92,12 @@ def test_mixed_launch_formats_4_and_5(tail_round):
         assert np.array_equal(y.cpu().numpy(), want), type
 
 
-def test_chosen_for_a_layer_of_a_few_rounds_and_equal_to_the_large_tile():
-    """At a benchmark size the library picks the mixed launch by itself (784 tiles of 128x128 on 256 compute units: three
-    whole rounds and a sixteenth); its output equals the plain 128x128 launch's."""
-    N, H, W, C, KN = 256, 14, 14, 256, 256
+@pytest.mark.parametrize("geometry,picked", [((256, 14, 14, 256, 256), 10), ((64, 28, 28, 512, 512), 11)])
+def test_chosen_for_a_layer_of_a_few_rounds_and_equal_to_the_large_tile(geometry, picked):
+    """At benchmark sizes the library picks the mixed launches by itself (N=256 14x14x256: 784 tiles of 128x128 on 256 compute
+    units, three whole rounds and a sixteenth; N=64 28x28x512: 784 tiles of 128x256); the output equals the plain 128x128
+    launch's."""
+    N, H, W, C, KN = geometry
     g = torch.Generator("cuda").manual_seed(3)
     x = torch.randn((N, H, W, C), generator=g, device="cuda")
     w = torch.randn((KN, 3, 3, C), generator=g, device="cuda")
@@ -114,4 +116,4 @@ def test_chosen_for_a_layer_of_a_few_rounds_and_equal_to_the_large_tile():
     lib.tab_internal_conv_shape.restype = ctypes.c_int
     lib.tab_internal_conv_shape.argtypes = [ctypes.c_int] * 6 + [ctypes.POINTER(ctypes.c_float)]
     cost = ctypes.c_float()
-    assert lib.tab_internal_conv_shape(3, N * H * W, KN, 36, 4, 0, ctypes.byref(cost)) == 10
+    assert lib.tab_internal_conv_shape(3, N * H * W, KN, 9 * (C // 64), C // 64, 0, ctypes.byref(cost)) == picked
