@@ -257,7 +257,7 @@ static int conv_packed(const int64_t *dev_QX, const int64_t *dev_QW, const int32
     a.div_ow = tab::make_div32((uint32_t)s.OW);
     a.div_tiles_m = tab::make_div32(1);
     a.tiles_n = 0;
-    a.xcd_share = 0; a.filter_tiles = 1; a.tail_big = 0;
+    a.xcd_share = 0; a.filter_tiles = 1; a.tail_big = 0; a.tail_chunks = 0;
     // A Y that fits the 256 MB last-level cache beside the operands but not the L2s is written through the caches
     // (the cache takes the stores faster than HBM: Y of 190-206 MB 1-11 % sooner); every other Y with non-temporal
     // stores: a smaller one leaves no dirty L2 to flush when the launch ends (7-25 % sooner), a larger one would only

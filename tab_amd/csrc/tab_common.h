@@ -75,6 +75,7 @@ struct ConvArgs {
     int filter_tiles;   // ceil(KN / BN), with div_filter_tiles, for that order
     Div32 div_filter_tiles;
     int tail_big;       // the mixed launch (conv_mfma_tail): workgroups that take whole 128x128 tiles; the rest take quarters
+    int tail_chunks;    // chunks of K of a quarter in that launch
     FastDiv div_pc, div_kw;
     Div32 div_pixels, div_ow;  // by OH*OW and OW: an output row's image and line
 };

@@ -168,18 +168,14 @@ __device__ __forceinline__ i32x8 expand_operand(uint32_t p0, uint32_t p1, const 
     return r;
 }
 
-// Words of K a kernel with chunks of KCH words multiplies: K rounded up to whole chunks (the words past K are zeros, which add
-// +64 each for binary x binary: the BNN bias counts them).
-template <int KCH>
-__device__ __forceinline__ int padded_words(const ConvArgs &p) { return (p.G + KCH - 1) / KCH * KCH; }
-
 // Epilogue shared by the matrix-core kernels: accumulator element 4*j + i of lane (kb, r) is
 // C[8*j + 4*kb + i][r] of the wave's 32x32 tile (mt, nt).  b_nonzero: BTN, bits set in the nonzero plane of
 // the k-positions this lane multiplied, per filter tile; partial: KS * 17 * 64 floats of LDS when the KS
-// waves of the workgroup hold partial sums of one tile.
+// waves of the workgroup hold partial sums of one tile; padded: words of K the kernel multiplied, K rounded up to whole
+// chunks (the words past K are zeros, which add +64 each for binary x binary: the BNN bias counts them).
 template <int TYPE, int TM, int TN, int KCH, int KS>
 __device__ __forceinline__ void conv_mfma_epilogue(const ConvArgs &p, f32x16 (&acc)[TM][TN], int (&b_nonzero)[TN], int wave_m0,
-                                                   int wave_n0, int lane, int ks, float *partial)
+                                                   int wave_n0, int lane, int ks, float *partial, int padded)
 {
     const int r = lane & 31, kb = lane >> 5;
     // btn of this lane's filters (BTN); loaded here rather than before the loop because the registers they would hold
@@ -209,7 +205,7 @@ __device__ __forceinline__ void conv_mfma_epilogue(const ConvArgs &p, f32x16 (&a
         const bool col_ok = col < p.KN;
         float bias = 0.f;
         if (TYPE == 2) bias = (float)btn_col[0] - (sum[4] + __shfl_xor(sum[4], 32, 64));
-        if (TYPE == 3) bias = (float)(p.num - 64 * padded_words<KCH>(p));
+        if (TYPE == 3) bias = (float)(p.num - 64 * padded);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const int m = wave_m0 + 8 * ks + 4 * kb + i;
@@ -236,7 +232,7 @@ __device__ __forceinline__ void conv_mfma_epilogue(const ConvArgs &p, f32x16 (&a
             const int nonzero = b_nonzero[nt] + __shfl_xor(b_nonzero[nt], 32, 64);
             bias = (float)(btn_col[nt] - nonzero);
         }
-        if (TYPE == 3) bias = (float)(p.num - 64 * padded_words<KCH>(p));
+        if (TYPE == 3) bias = (float)(p.num - 64 * padded);
         // kNoFilter + any offset inside the tile stays out of range without wrapping
         const uint32_t lane_off = col < p.KN ? (uint32_t)(4 * kb) * row_bytes + (uint32_t)col * 4u : kNoFilter;
         auto store_tiles = [&](auto policy) {
@@ -266,7 +262,7 @@ __device__ __forceinline__ void conv_mfma_epilogue(const ConvArgs &p, f32x16 (&a
 // handed to the lanes that need it through `exchange`, 32*TN dwords of LDS private to the wave.
 template <int TYPE, int TM, int TN, int KCH>
 __device__ __forceinline__ void conv_mfma_epilogue_packed(const ConvArgs &p, f32x16 (&acc)[TM][TN], int (&b_nonzero)[TN], int wave_m0,
-                                                          int wave_n0, int lane, uint32_t *exchange)
+                                                          int wave_n0, int lane, uint32_t *exchange, int padded)
 {
     const int r = lane & 31, kb = lane >> 5;
     const long rows_left = (long)p.M - wave_m0;
@@ -297,7 +293,7 @@ __device__ __forceinline__ void conv_mfma_epilogue_packed(const ConvArgs &p, f32
             if (TYPE == 2) v = *reinterpret_cast<const u32x4 *>(exchange + nt * 32 + 8 * j + 4 * kb);
 #pragma unroll
             for (int i = 0; i < 4; i++)
-                bias[nt][4 * j + i] = TYPE == 2 ? __uint_as_float(v[i]) : (TYPE == 3 ? (float)(p.num - 64 * padded_words<KCH>(p)) : 0.f);
+                bias[nt][4 * j + i] = TYPE == 2 ? __uint_as_float(v[i]) : (TYPE == 3 ? (float)(p.num - 64 * padded) : 0.f);
         }
 
     auto pack_rows = [&](auto out_bits_constant) {
@@ -543,9 +539,9 @@ __attribute__((amdgpu_waves_per_eu(mfma_waves_per_eu(WM, TM, TN, conv_mfma_lds_b
 
     scale_ternary_sums<TYPE>(acc);
     if constexpr (PACKED)  // (the chunk loop ends on a barrier: the operand buffers are free for BTN's exchange of biases)
-        conv_mfma_epilogue_packed<TYPE, TM, TN, KCH>(p, acc, b_nonzero, wave_m0, wave_n0, lane, lds + wave * (32 * TN));
+        conv_mfma_epilogue_packed<TYPE, TM, TN, KCH>(p, acc, b_nonzero, wave_m0, wave_n0, lane, lds + wave * (32 * TN), p.nchunks * KCH);
     else
-        conv_mfma_epilogue<TYPE, TM, TN, KCH, KS>(p, acc, b_nonzero, wave_m0, wave_n0, lane, ks, partial);
+        conv_mfma_epilogue<TYPE, TM, TN, KCH, KS>(p, acc, b_nonzero, wave_m0, wave_n0, lane, ks, partial, p.nchunks * KCH);
 }
 
 // Chunk length for G words: 1..4, the one with the least padded work (a barrier is priced as half a

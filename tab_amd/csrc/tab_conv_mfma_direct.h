@@ -75,9 +75,9 @@ constexpr int conv_mfma_direct_lds_dwords()
 }
 
 // One tile of Y, by the whole workgroup: tile (tile_m, tile_n) of the launch's BM x BN grid, operands through the
-// workgroup's LDS `lds` (conv_mfma_direct_lds_dwords<...>() dwords).
+// workgroup's LDS `lds` (conv_mfma_direct_lds_dwords<...>() dwords); nchunks = ceil(G / KCH), from the host.
 template <int TYPE, int WM, int WN, int TM, int TN, int KCH, bool PACKED, int KS, int ARUN>
-__device__ __forceinline__ void conv_mfma_direct_tile(const ConvArgs &p, uint32_t *lds, int tile_m, int tile_n)
+__device__ __forceinline__ void conv_mfma_direct_tile(const ConvArgs &p, uint32_t *lds, int tile_m, int tile_n, int nchunks)
 {
     static_assert(WM * WN * KS * 64 == kConvThreads && KCH % (2 * KS) == 0, "four waves, whole pairs of words per wave group");
     constexpr int PAIRS = KCH / 2;
@@ -91,7 +91,6 @@ __device__ __forceinline__ void conv_mfma_direct_tile(const ConvArgs &p, uint32_
     constexpr int A_RUN = ARUN ? ARUN : granule_run(PA, APL), B_RUN = granule_run(PB, BPL);
     static_assert(BM % 64 == 0 && BN % 64 == 0, "one wave instruction moves 64 / RUN rows of one run");
     static_assert(PA % A_RUN == 0, "whole runs");
-    const int nchunks = (p.G + KCH - 1) / KCH;  // (the split-K shapes fetch the words past K as zeros)
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -398,9 +397,9 @@ __device__ __forceinline__ void conv_mfma_direct_tile(const ConvArgs &p, uint32_
                     if (TYPE == 2) nonzero[0] += __float_as_int(src[16 * 64 + lane]);
                 }
                 if constexpr (PACKED)
-                    conv_mfma_epilogue_packed<TYPE, 1, 1, KCH>(p, sum, nonzero, wave_m0 + mt * 32, wave_n0 + nt * 32, lane, exchange);
+                    conv_mfma_epilogue_packed<TYPE, 1, 1, KCH>(p, sum, nonzero, wave_m0 + mt * 32, wave_n0 + nt * 32, lane, exchange, nchunks * KCH);
                 else
-                    conv_mfma_epilogue<TYPE, 1, 1, KCH, 1>(p, sum, nonzero, wave_m0 + mt * 32, wave_n0 + nt * 32, lane, 0, nullptr);
+                    conv_mfma_epilogue<TYPE, 1, 1, KCH, 1>(p, sum, nonzero, wave_m0 + mt * 32, wave_n0 + nt * 32, lane, 0, nullptr, nchunks * KCH);
             }
             if (round + 1 < NT / RT) __syncthreads();  // the parts are read before the next round overwrites them
         }
@@ -408,9 +407,9 @@ __device__ __forceinline__ void conv_mfma_direct_tile(const ConvArgs &p, uint32_
         // BTN hands its biases round through LDS: not before every wave has read its last operands (the pipelined
         // loop reads the zeros past the last chunk after the chunk's barrier and counts their nonzero weights)
         if (TYPE == 2) __syncthreads();
-        conv_mfma_epilogue_packed<TYPE, TM, TN, KCH>(p, acc, b_nonzero, wave_m0, wave_n0, lane, lds + wave * (32 * TN));
+        conv_mfma_epilogue_packed<TYPE, TM, TN, KCH>(p, acc, b_nonzero, wave_m0, wave_n0, lane, lds + wave * (32 * TN), nchunks * KCH);
     } else {
-        conv_mfma_epilogue<TYPE, TM, TN, KCH, 1>(p, acc, b_nonzero, wave_m0, wave_n0, lane, 0, nullptr);
+        conv_mfma_epilogue<TYPE, TM, TN, KCH, 1>(p, acc, b_nonzero, wave_m0, wave_n0, lane, 0, nullptr, nchunks * KCH);
     }
 }
 
@@ -421,7 +420,7 @@ __attribute__((amdgpu_waves_per_eu(mfma_waves_per_eu(KS > 1 ? 1 : WM, TM, TN, 4 
     __shared__ __attribute__((aligned(16))) uint32_t lds[conv_mfma_direct_lds_dwords<TYPE, WM, WN, TM, TN, KCH, KS>()];
     int tile_m, tile_n;
     if (!tile_of_workgroup(p, tile_m, tile_n)) return;
-    conv_mfma_direct_tile<TYPE, WM, WN, TM, TN, KCH, PACKED, KS, ARUN>(p, lds, tile_m, tile_n);
+    conv_mfma_direct_tile<TYPE, WM, WN, TM, TN, KCH, PACKED, KS, ARUN>(p, lds, tile_m, tile_n, p.nchunks);
 }
 
 // Mixed launch for grids of a few rounds of the chip: a launch lasts as long as its busiest CU, and with T tiles on C CUs that
@@ -443,14 +442,14 @@ __global__ __launch_bounds__(kConvThreads) __attribute__((amdgpu_waves_per_eu(TN
         // XCD-aware order over the whole tiles, as in tile_of_workgroup
         const uint32_t logical = b < 8u * (uint32_t)p.xcd_share ? (b & 7u) * (uint32_t)p.xcd_share + (b >> 3) : b;
         const int tile_m = (int)div32(logical, p.div_filter_tiles);
-        conv_mfma_direct_tile<TYPE, 2, 2, 2, TNB, KCH, PACKED, 1, 0>(p, lds, tile_m, (int)logical - tile_m * p.filter_tiles);
+        conv_mfma_direct_tile<TYPE, 2, 2, 2, TNB, KCH, PACKED, 1, 0>(p, lds, tile_m, (int)logical - tile_m * p.filter_tiles, p.nchunks);
     } else {
         constexpr uint32_t PIECES = 2 * TNB;  // 64x64 quarters of a whole tile
         const uint32_t j = b - (uint32_t)p.tail_big, t = (uint32_t)p.tail_big + j / PIECES, q = j % PIECES;
         const int big_m = (int)div32(t, p.div_filter_tiles), big_n = (int)t - big_m * p.filter_tiles;
         const int tile_m = 2 * big_m + (int)(q & 1u), tile_n = TNB * big_n + (int)(q >> 1);
         if (tile_m * 64 >= p.M || tile_n * 64 >= p.KN) return;  // a quarter wholly past the edge of Y
-        conv_mfma_direct_tile<TYPE, 1, 1, 2, 2, 8, PACKED, 4, ARUN>(p, lds, tile_m, tile_n);
+        conv_mfma_direct_tile<TYPE, 1, 1, 2, 2, 8, PACKED, 4, ARUN>(p, lds, tile_m, tile_n, p.tail_chunks);
     }
 }
 
@@ -459,6 +458,7 @@ hipError_t launch_mfma_tail_run(ConvArgs a, long blocks, hipStream_t stream)
 {
     a.kcw = KCH;
     a.nchunks = a.G / KCH;
+    a.tail_chunks = (a.G + 7) / 8;  // the quarters' chunks of eight words, the last one padded with zeros
     if (a.qy != nullptr) {
         if constexpr (TYPE <= 3)
             conv_mfma_tail<TYPE, KCH, ARUN, true, TNB><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
