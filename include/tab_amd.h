@@ -196,7 +196,8 @@ int tab_conv2d_packed(const int64_t *dev_QX, const int64_t *dev_QW, const int32_
  *   dev_out_ths fp32 [>=N]: threshold for the outputs of image n
  *   dev_QY      int64 [N*OH*OW*ceil(KN/64)*out_bitwidth], aligned to a whole packed element
  *               (8*out_bitwidth bytes); every element is written
- * Types 0..3 only.
+ * All six types; types 4 and 5 take dev_QX / dev_QW as tab_conv2d_packed does, and their output, too, is packed as
+ * tab_quantize packs it (bit planes for a following layer of types 0..3).
  */
 int tab_conv2d_packed_out(const int64_t *dev_QX, const int64_t *dev_QW, const int32_t *dev_btn,
                           int type, int padding1, int padding2, int stride1, int stride2, int N,

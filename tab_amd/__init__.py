@@ -315,12 +315,10 @@ def Conv2dPackedOut(QX, QW, btn, type, padding1, padding2, stride1, stride2, N, 
     _check_dtype(out_thresholds, torch.float32, "out_thresholds")
     (type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW, out_bitwidth) = (
         int(v) for v in (type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW, out_bitwidth))
-    if type not in (0, 1, 2, 3):
-        raise RuntimeError(f"packed output exists for types 0..3 only, got {type}")
     OH, OW = _conv_checks(QW, btn, type, N, H, W, C, KN, KH, KW, padding1, padding2, stride1, stride2)
-    abits = 2 if type < 2 else 1
-    if QX.numel() != N * H * W * packed_channels(C) * abits:
-        raise RuntimeError(f"QX has {QX.numel()} words, type {type} expects N*H*W*PC*{abits}")
+    awords = operand_words(type, 0, C)
+    if QX.numel() != N * H * W * awords:
+        raise RuntimeError(f"QX has {QX.numel()} words, type {type} expects N*H*W*{awords}")
     if out_thresholds.numel() < N:
         raise RuntimeError(f"out_thresholds has {out_thresholds.numel()} elements, need N={N}")
     if out_bitwidth not in (1, 2):

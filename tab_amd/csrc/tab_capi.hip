@@ -228,7 +228,6 @@ static int conv_packed(const int64_t *dev_QX, const int64_t *dev_QW, const int32
     rc = check_conv_pointers(s, type, dev_QX, dev_QW, dev_btn, dev_Y, dev_QY);
     if (rc != TAB_OK) return rc;
     if (dev_QY) {
-        if (type > 3) return fail(TAB_ERR_BAD_ARGUMENT, "packed output exists for types 0..3 only, got %d", type);
         if (out_bitwidth != 1 && out_bitwidth != 2)
             return fail(TAB_ERR_BAD_ARGUMENT, "out_bitwidth must be 1 or 2, got %d", out_bitwidth);
         if (!dev_out_ths) return fail(TAB_ERR_BAD_ARGUMENT, "null device pointer");

@@ -432,7 +432,7 @@ __global__ __launch_bounds__(kConvThreads)
 __attribute__((amdgpu_waves_per_eu(mfma_waves_per_eu(WM, TM, TN, conv_mfma_lds_bytes<TYPE, WM, WN, TM, TN, KCH, INTAP, KS>())))) void conv_mfma(const ConvArgs p)
 {
     static_assert(WM * WN * KS * 64 == kConvThreads, "four waves");
-    static_assert(!PACKED || (KS == 1 && TYPE <= 3), "packed output: whole tiles per wave, types 0..3");
+    static_assert(!PACKED || KS == 1, "packed output: whole tiles per wave");
     static_assert(KCH % KS == 0 && (KS == 1 || (TM == 1 && TN == 1)), "k-split waves share one 32x32 tile");
     constexpr int WPW = KCH / KS;  // words of a chunk each wave multiplies
     constexpr int APL = Planes<TYPE>::A, BPL = Planes<TYPE>::B;
@@ -566,10 +566,10 @@ hipError_t launch_mfma_tile(ConvArgs a, hipStream_t stream)
     const long blocks = order_workgroups<Planes<TYPE>::A>(a, (a.KN + BN - 1) / BN);
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
     if (a.qy != nullptr) {
-        if constexpr (TYPE <= 3 && KS == 1)
+        if constexpr (KS == 1)
             conv_mfma<TYPE, WM, WN, TM, TN, KCH, INTAP, KS, true><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
         else
-            return hipErrorInvalidValue;  // no packed output for types 4 and 5, nor from the k-split 32x32 shape
+            return hipErrorInvalidValue;  // no packed output from the k-split 32x32 shape
     } else {
         conv_mfma<TYPE, WM, WN, TM, TN, KCH, INTAP, KS><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
     }

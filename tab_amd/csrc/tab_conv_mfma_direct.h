@@ -460,10 +460,7 @@ hipError_t launch_mfma_tail_run(ConvArgs a, long blocks, hipStream_t stream)
     a.nchunks = a.G / KCH;
     a.tail_chunks = (a.G + 7) / 8;  // the quarters' chunks of eight words, the last one padded with zeros
     if (a.qy != nullptr) {
-        if constexpr (TYPE <= 3)
-            conv_mfma_tail<TYPE, KCH, ARUN, true, TNB><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
-        else
-            return hipErrorInvalidValue;  // no packed output for types 4 and 5
+        conv_mfma_tail<TYPE, KCH, ARUN, true, TNB><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
     } else {
         conv_mfma_tail<TYPE, KCH, ARUN, false, TNB><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
     }
@@ -540,10 +537,7 @@ hipError_t launch_mfma_direct(ConvArgs a, hipStream_t stream)
     const long blocks = order_workgroups<Planes<TYPE>::A>(a, (a.KN + BN - 1) / BN);
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
     if (a.qy != nullptr) {
-        if constexpr (TYPE <= 3)
-            conv_mfma_direct<TYPE, WM, WN, TM, TN, KCH, true, KS, ARUN><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
-        else
-            return hipErrorInvalidValue;  // no packed output for types 4 and 5
+        conv_mfma_direct<TYPE, WM, WN, TM, TN, KCH, true, KS, ARUN><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
     } else {
         conv_mfma_direct<TYPE, WM, WN, TM, TN, KCH, false, KS, ARUN><<<dim3((unsigned)blocks), dim3(kConvThreads), 0, stream>>>(a);
     }

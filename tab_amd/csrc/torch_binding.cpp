@@ -203,7 +203,6 @@ torch::Tensor TAB_Conv2dPackedOut(torch::Tensor QX, torch::Tensor QW, torch::Ten
     CHECK_DTYPE(QW, torch::kInt64);
     CHECK_DTYPE(btn, torch::kInt32);
     CHECK_DTYPE(out_thresholds, torch::kFloat32);
-    TORCH_CHECK(type >= 0 && type <= 3, "packed output exists for types 0..3 only, got ", type);
     TORCH_CHECK(out_bitwidth == 1 || out_bitwidth == 2, "out_bitwidth must be 1 or 2, got ", out_bitwidth);
     const auto [OH, OW] = check_conv(QW, btn, type, padding1, padding2, stride1, stride2, N, H, W, C, KN, KH, KW);
     const int awords = tab_operand_words(type, 0, C);

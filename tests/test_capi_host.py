@@ -85,9 +85,10 @@ def test_c_abi_rejects_bad_arguments_without_launching():
     assert out(ths=None) == -1
     assert out(qy=None) == -1
     assert out(qy=p + 8, bits=2) == -1 and b"aligned" in lib.tab_last_error()
-    # the CPU-only types: no packed output; type 4 bounds K so that 9 * 64 * K words stays below 2^24
-    assert lib.tab_conv2d_packed_out(p, p, p, 4, 1, 1, 1, 1, 1, 8, 8, 64, 4, 3, 3, p, 1, p, None) == -1
-    assert b"types 0..3" in lib.tab_last_error()
+    # the CPU-only types: packed output takes the same checks; type 4 bounds K so that 9 * 64 * K words stays below 2^24
+    assert lib.tab_conv2d_packed_out(p, p, p, 4, 1, 1, 1, 1, 1, 8, 8, 64, 4, 3, 3, p, 3, p, None) == -1
+    assert b"out_bitwidth" in lib.tab_last_error()
+    assert lib.tab_conv2d_packed_out(p, p, p, 5, 1, 1, 1, 1, 1, 8, 8, 64, 4, 3, 3, None, 1, p, None) == -1
     assert lib.tab_conv2d_packed(p, p, p, 4, 0, 0, 1, 1, 1, 4, 4, 64 * 29200, 4, 1, 1, p, None) == -2
     assert b"exact accumulation" in lib.tab_last_error()
     assert lib.tab_conv2d_packed(p, p, p, 5, 0, 0, 1, 1, 1, 4, 4, 32 * 65536, 4, 1, 1, p, None) == -2

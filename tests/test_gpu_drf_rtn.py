@@ -105,6 +105,37 @@ def test_conv2d_packed_any_bits_every_tile(type, kernel, restore_kernel_choice):
         assert np.array_equal(got, want), f"max |diff| = {np.abs(got - want).max()}"
 
 
+PACKED_OUT_KERNELS = [(tab_amd.CONV_AUTO, -1)] + [(tab_amd.CONV_MATRIX, t) for t in (0, 1, 2, 4, 5, 6, 8, 9, 10, 11)]
+
+
+@pytest.mark.parametrize("type", [4, 5])
+@pytest.mark.parametrize("kernel", PACKED_OUT_KERNELS)
+def test_packed_output_every_tile(type, kernel, restore_kernel_choice):
+    """Conv2dPackedOut for the two CPU-path types: the conv's outputs thresholded and packed in the epilogue as Quantize packs
+    them (1- and 2-bit planes), against the oracle's conv followed by the oracle's quantizer.  Thresholds sit inside the range
+    of the sums, on values the integer sums hit (ties)."""
+    tab_amd.set_conv_kernel(*kernel)
+    for case in [(2, 9, 6, 70, 5, 3, 3, 1, 0, 1, 2), (2, 12, 12, 192, 130, 3, 3, 1, 1, 1, 1), (3, 9, 9, 512, 72, 3, 3, 1, 1, 2, 2),
+                 (2, 10, 10, 256, 200, 3, 3, 1, 1, 1, 1)]:
+        N, H, W, C, KN, KH, KW, p1, p2, s1, s2 = case
+        print(f"[case] Conv2dPackedOut {TYPE_NAMES[type]} kernel={kernel} {case}", flush=True)
+        rng = np.random.default_rng(type * 7 + C)
+        qx = _rand_words(rng, (N, H, W, tab_amd.operand_words(type, 0, C)))
+        qw = _rand_words(rng, (KN, KH, KW, tab_amd.operand_words(type, 1, C)))
+        y = oracle.conv2d_packed(qx, qw, None, type, p1, p2, s1, s2, N, H, W, C, KN, KH, KW)
+        OH, OW = tab_amd.out_shape(H, W, KH, KW, p1, p2, s1, s2)
+        y = np.ascontiguousarray(y).reshape(N, OH, OW, KN)
+        btn = torch.zeros(KN, dtype=torch.int32, device="cuda")
+        for out_bits in (1, 2):
+            # per image: the median of its sums (binary: about half the bits set) or of their magnitudes (ternary)
+            ths = np.array([np.median(y[n]) if out_bits == 1 else np.median(np.abs(y[n])) for n in range(N)], dtype=np.float32)
+            want, _ = oracle.quantize(y, ths, out_bits, N, OH, OW, KN)
+            got = tab_amd.Conv2dPackedOut(torch.from_numpy(qx).cuda(), torch.from_numpy(qw).cuda(), btn, type, p1, p2, s1, s2,
+                                          N, H, W, C, KN, KH, KW, torch.from_numpy(ths).cuda(), out_bits)
+            torch.cuda.synchronize()
+            assert np.array_equal(got.cpu().numpy(), want), f"{TYPE_NAMES[type]} {case} out_bits={out_bits}"
+
+
 @pytest.mark.parametrize("type", [4, 5])
 def test_saturated_operands_stay_exact(type):
     """All-ones words: every product takes its largest value (9 per bit for type 4), the sums the

@@ -148,5 +148,11 @@ def test_every_extension_entry_point_equals_ctypes_front_end():
         assert np.array_equal(ya.cpu().numpy(), want)
         QX = TAB.QuantizeFormat(xs, x_t, type, N, H, W, C)
         assert torch.equal(TAB.Conv2dPacked(QX, QWa, btn, type, 1, 1, 2, 1, N, H, W, C, KN, 3, 3), ya)
-    with pytest.raises(RuntimeError, match="types 0..3 only"):
-        TAB.Conv2dPackedOut(QX, QWa, btn, 4, 1, 1, 2, 1, N, H, W, C, KN, 3, 3, x_t, 1)
+        # packed output for these types too: both front ends agree with quantizing the fp32 result
+        OH, OW = tab_amd.out_shape(H, W, 3, 3, 1, 1, 2, 1)
+        out_t = torch.full((N,), float(ya.abs().median()), device="cuda")
+        for out_bits in (1, 2):
+            qa = TAB.Conv2dPackedOut(QX, QWa, btn, type, 1, 1, 2, 1, N, H, W, C, KN, 3, 3, out_t, out_bits)
+            qb = tab_amd.Conv2dPackedOut(QX, QWa, btn, type, 1, 1, 2, 1, N, H, W, C, KN, 3, 3, out_t, out_bits)
+            want_q, _ = tab_amd.Quantize(ya.view(N, OH, OW, KN), out_t, out_bits, N, OH, OW, KN)
+            assert torch.equal(qa, qb) and torch.equal(qa.reshape(want_q.shape), want_q)
