@@ -810,10 +810,12 @@ def main():
             vgg_ms += k_ms
             vgg_call_ms += c_ms
             vgg.append({"layer": layer_name(32, lay), "conv_kernel_us": round(k_ms * 1e3, 1), "call_us": round(c_ms * 1e3, 1),
-                        "conv_kernel_tops": round(L.ops / k_ms / 1e9, 1), "rows_checked": g["rows_checked"],
+                        "conv_kernel_tops": round(L.ops / k_ms / 1e9, 1),
+                        "frac_mfma_peak": round(L.ops / k_ms / 1e9 / MFMA_FP4_PEAK_TOPS, 4), "rows_checked": g["rows_checked"],
                         "cpu_ms_extrapolated": cpu["cpu_ms"]})
             del L
         result["vgg16_tnn_N32"] = {"conv_kernel_tops": round(vgg_ops / vgg_ms / 1e9, 1),
+                                   "frac_mfma_peak": round(vgg_ops / vgg_ms / 1e9 / MFMA_FP4_PEAK_TOPS, 4),
                                    "call_tops": round(vgg_ops / vgg_call_ms / 1e9, 1), "bit_exact_vs_cpu": vgg_ok,
                                    "cpu_tops_extrapolated_from_4_images": round(vgg_ops / vgg_cpu_ms / 1e9, 3), "layers": vgg}
         result["all_gates_bit_exact"] = bool(
